@@ -1,0 +1,211 @@
+"""Seeded synthetic inputs for the sparse-attention path.
+
+Host-side counterparts of the reference drivers' generators (paths relative to
+the reference tree):
+
+* ``gen_block_table``   examples/models/deepseek_v32_exp/
+  deepseekv32_sparse_flash_attention_quant.py:257-295 and
+  deepseekv32_lightning_indexer_quant.py:83-116 (random permutation of the
+  physical blocks, ``-1`` in unused table slots)
+* ``gen_sfa_inputs``    ...sparse_flash_attention_quant.py:298-388 (tensor names,
+  shapes and layouts of the operator inputs; index rows are a random subset of
+  the valid positions, or ``arange`` when fewer than ``topk`` exist)
+* ``gen_indexer_inputs`` ...lightning_indexer_quant.py:119-181
+
+Unlike the reference (global ``torch.manual_seed`` plus an unseeded
+``np.random.permutation``) every generator here draws from an explicit
+``torch.Generator`` so that a seed fully determines the inputs.
+
+Value distributions follow the benchmark configurations: q ~ N(0,1) bf16, latent
+KV int8 uniform in [-127,127] with fp32 scales uniform in [0.005,0.02] (four per
+token), rope K ~ N(0,1) bf16; indexer q/k int8 uniform in [-127,127], per-token
+scales, per-head weights N(0,1)/8.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import torch
+
+BLOCK_SIZE = 128
+KV_LORA_RANK = 512
+ROPE_DIM = 64
+IDX_HEADS = 64
+IDX_DIM = 128
+
+
+def gen_block_table(act_seq: Sequence[int], block_size: int, generator: Optional[torch.Generator] = None,
+                    shuffle: bool = True, max_kv: Optional[int] = None):
+    """Returns (block_num, block_table [B, ceil(max_kv/bs)] int32 with -1 padding)."""
+    act = [int(a) for a in act_seq]
+    per = [math.ceil(a / block_size) for a in act]
+    block_num = sum(per)
+    mb = math.ceil((max_kv if max_kv is not None else max(act + [1])) / block_size)
+    mb = max(mb, 1)
+    if shuffle:
+        ids = torch.randperm(block_num, generator=generator).to(torch.int32)
+    else:
+        ids = torch.arange(block_num, dtype=torch.int32)
+    table = -torch.ones([len(act), mb], dtype=torch.int32)
+    pos = 0
+    for i, n in enumerate(per):
+        table[i, :n] = ids[pos:pos + n]
+        pos += n
+    return block_num, table
+
+
+def gen_topk_indices(act_seq: Sequence[int], s1: int, topk: int, generator: torch.Generator,
+                     causal: bool = True) -> torch.Tensor:
+    """[B*S1, topk] int32.  Row (b, s) holds ``cur = min(max(act-S1+1+s,0), topk)`` valid
+    entries: a random subset of the positions ``0 .. act-S1+s`` when more than
+    ``topk`` exist, else ``arange``; the remainder is -1 (what the indexer pads with)."""
+    b = len(act_seq)
+    out = -torch.ones([b * s1, topk], dtype=torch.int32)
+    for bi, act in enumerate(act_seq):
+        for s in range(s1):
+            eff = int(act) - (s1 - 1 - s) if causal else int(act)
+            eff = max(eff, 0)
+            if eff <= topk:
+                out[bi * s1 + s, :eff] = torch.arange(eff, dtype=torch.int32)
+            else:
+                out[bi * s1 + s] = torch.randperm(eff, generator=generator)[:topk].to(torch.int32)
+    return out
+
+
+@dataclass
+class SfaInputs:
+    b: int
+    s1: int
+    n_q: int
+    n_kv: int
+    topk: int
+    block_size: int
+    block_num: int
+    max_blocknum_perbatch: int
+    softmax_scale: float
+    actual_seq: List[int]
+    query_nope: torch.Tensor      # [B*S1*Nq, 512] bf16
+    query_rope: torch.Tensor      # [B*S1*Nq, 64]  bf16
+    key_nope_2d: torch.Tensor     # [NB*bs, 512]   int8
+    key_rope_2d: torch.Tensor     # [NB*bs, 64]    bf16
+    k_nope_scales: torch.Tensor   # [NB*bs, 4]     fp32
+    topk_indices: torch.Tensor    # [B*S1, topk]   int32
+    block_table: torch.Tensor     # [B, MB]        int32
+    kv_act_seqs: torch.Tensor     # [B]            int32
+
+    def q_bsnd(self) -> torch.Tensor:
+        """[B,S1,Nq,576] view (nope ‖ rope) as the goldens take it."""
+        q = torch.cat([self.query_nope, self.query_rope], dim=-1)
+        return q.reshape(self.b, self.s1, self.n_q, -1)
+
+    def operator_tensors(self):
+        return (self.query_nope, self.query_rope, self.key_nope_2d, self.key_rope_2d, self.k_nope_scales,
+                self.topk_indices, self.block_table, self.kv_act_seqs)
+
+    def to(self, device) -> "SfaInputs":
+        kw = dict(self.__dict__)
+        for k, v in kw.items():
+            if isinstance(v, torch.Tensor):
+                kw[k] = v.to(device)
+        return SfaInputs(**kw)
+
+
+def gen_sfa_inputs(b: int, s1: int, n_q: int, actual_seq: Sequence[int], topk: int = 2048, seed: int = 0,
+                   block_size: int = BLOCK_SIZE, shuffle_table: bool = True,
+                   topk_indices: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
+                   block_num: Optional[int] = None) -> SfaInputs:
+    g = torch.Generator().manual_seed(seed)
+    act = [int(a) for a in actual_seq]
+    assert len(act) == b
+    if block_table is None:
+        block_num, block_table = gen_block_table(act, block_size, g, shuffle=shuffle_table)
+    rows = block_num * block_size
+    t = b * s1
+    q_nope = torch.randn([t * n_q, KV_LORA_RANK], generator=g).to(torch.bfloat16)
+    q_rope = torch.randn([t * n_q, ROPE_DIM], generator=g).to(torch.bfloat16)
+    kn = torch.randint(-127, 128, [rows, KV_LORA_RANK], generator=g, dtype=torch.int8)
+    kr = torch.randn([rows, ROPE_DIM], generator=g).to(torch.bfloat16)
+    scales = 0.005 + 0.015 * torch.rand([rows, 4], generator=g, dtype=torch.float32)
+    if topk_indices is None:
+        topk_indices = gen_topk_indices(act, s1, topk, g)
+    d = KV_LORA_RANK + ROPE_DIM
+    return SfaInputs(b=b, s1=s1, n_q=n_q, n_kv=1, topk=topk, block_size=block_size, block_num=block_num,
+                     max_blocknum_perbatch=block_table.shape[1], softmax_scale=d ** -0.5, actual_seq=act,
+                     query_nope=q_nope, query_rope=q_rope, key_nope_2d=kn, key_rope_2d=kr, k_nope_scales=scales,
+                     topk_indices=topk_indices.reshape(t, topk).contiguous(), block_table=block_table,
+                     kv_act_seqs=torch.tensor(act, dtype=torch.int32))
+
+
+@dataclass
+class IndexerInputs:
+    b: int
+    s1: int
+    selected_count: int
+    block_size: int
+    block_num: int
+    act_seq: List[int]
+    idx_query: torch.Tensor        # [T, 64, 128]       int8
+    idx_query_scale: torch.Tensor  # [T, 64]            fp16 | fp32
+    idx_key_cache: torch.Tensor    # [NB, bs, 1, 128]   int8
+    idx_key_scale: torch.Tensor    # [NB, bs, 1]        fp16 | fp32
+    idx_weight: torch.Tensor       # [T, 64]            fp16 | bf16
+    act_seq_key: torch.Tensor      # [B]                int32
+    block_table: torch.Tensor      # [B, MB]            int32
+    topk_res: torch.Tensor = field(default=None)  # [T, 1, k] int32 output buffer
+
+    def operator_tensors(self):
+        return (self.idx_query, self.idx_query_scale, self.idx_key_cache, self.idx_key_scale, self.idx_weight,
+                self.act_seq_key, self.block_table, self.topk_res)
+
+    def to(self, device) -> "IndexerInputs":
+        kw = dict(self.__dict__)
+        for k, v in kw.items():
+            if isinstance(v, torch.Tensor):
+                kw[k] = v.to(device)
+        return IndexerInputs(**kw)
+
+
+def gen_indexer_inputs(b: int, s1: int, act_seq: Sequence[int], selected_count: int = 2048, seed: int = 0,
+                       variant: str = "fp16", block_size: int = BLOCK_SIZE, shuffle_table: bool = True,
+                       block_table: Optional[torch.Tensor] = None, block_num: Optional[int] = None,
+                       n_heads: int = IDX_HEADS, head_dim: int = IDX_DIM) -> IndexerInputs:
+    """``variant='fp16'``: fp16 scales and weights (the reference's dtypes);
+    ``variant='fp32'``: fp32 scales and bf16 weights (the benchmark configuration)."""
+    g = torch.Generator().manual_seed(seed)
+    act = [int(a) for a in act_seq]
+    if block_table is None:
+        block_num, block_table = gen_block_table(act, block_size, g, shuffle=shuffle_table)
+    t = b * s1
+    q = torch.randint(-127, 128, [t, n_heads, head_dim], generator=g, dtype=torch.int8)
+    k = torch.randint(-127, 128, [block_num, block_size, 1, head_dim], generator=g, dtype=torch.int8)
+    qs = 0.005 + 0.015 * torch.rand([t, n_heads], generator=g, dtype=torch.float32)
+    ks = 0.005 + 0.015 * torch.rand([block_num, block_size, 1], generator=g, dtype=torch.float32)
+    w = torch.randn([t, n_heads], generator=g, dtype=torch.float32) / 8
+    if variant == "fp16":
+        qs, ks, w = qs.to(torch.float16), ks.to(torch.float16), w.to(torch.float16)
+    elif variant == "fp32":
+        w = w.to(torch.bfloat16)
+    else:
+        raise ValueError(f"unknown variant {variant!r}")
+    return IndexerInputs(b=b, s1=s1, selected_count=selected_count, block_size=block_size, block_num=block_num,
+                         act_seq=act, idx_query=q, idx_query_scale=qs, idx_key_cache=k, idx_key_scale=ks,
+                         idx_weight=w, act_seq_key=torch.tensor(act, dtype=torch.int32), block_table=block_table,
+                         topk_res=torch.zeros([t, 1, selected_count], dtype=torch.int32))
+
+
+def config_lengths(cfg: int, seed: int = 0) -> List[int]:
+    """Per-sequence KV lengths of the benchmark configurations 0-4."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    if cfg == 0:
+        return [4096]
+    if cfg == 1:
+        return [32768] * 4
+    if cfg == 2:
+        return torch.randint(8192, 65537, [32], generator=g).tolist()
+    if cfg == 3:
+        return torch.randint(4096, 32769, [64], generator=g).tolist()
+    if cfg == 4:
+        return [4096]
+    raise ValueError(cfg)
