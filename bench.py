@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized DeepSeek-V3.2 sparse-attention decode path on one MI355X.
+
+A step is one pass of sparse flash attention over one batch: B=32 sequences, one query token each,
+128 heads, d=576/512, top-k 2048 chosen by the lightning indexer, paged int8 latent KV with per-token
+scales, per-sequence KV lengths drawn from 8192..65536.  All inputs are resident in HBM before the
+timed region.  Prints ONE JSON line:
+
+  value          query tokens per second (B / step time) over K timed steps
+  roofline       achieved bf16 matrix throughput of the attention launch = algorithmic flops per step
+                 / average launch duration from HIP events on the launch stream, against 2.5 PFLOP/s;
+                 the HBM-side figure (algorithmic bytes / same duration, against 8 TB/s) is in
+                 "roofline_hbm" because the shape sits at the ridge of the two
+  indexer        time of one lightning-indexer pass (score + select) on the same batch and on the
+                 indexer-only configuration (B=4, KV 32768), with its HBM fraction
+  cpu_baseline   the scalar C statement of the golden, all host threads, on a bounded sample of the
+                 same batch
+
+To keep a step from being served out of the 256 MB memory-side cache, steps rotate over ROT
+different selections (different indexer queries over the same caches).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0
+PEAK_HBM_GBS = 8000.0
+ROT = 8
+
+
+def sfa_algorithmic_work(cur_seqs, n_heads=128):
+    """Bytes and flops of one step: per query row with n selected keys,
+    n*(512 + 128 + 16) KV + n*4 indices + 4 per page touched (<= n, counted as min(n, pages)) +
+    heads*576*2 query + heads*512*2 output; flops = 2*heads*n*(576+512)."""
+    byt = flops = 0
+    for n in cur_seqs:
+        byt += n * (512 + 128 + 16) + n * 4 + 4 * n + n_heads * 576 * 2 + n_heads * 512 * 2
+        flops += 2 * n_heads * n * (576 + 512)
+    return byt, flops
+
+
+def indexer_algorithmic_bytes(lengths, k_scale_bytes, k=2048):
+    """Per query token over L keys: L*(128 + scale) + 64*128 query + 64*(scale+weight) + 4 per page + k*4 out."""
+    return sum(L * (128 + k_scale_bytes) + 64 * 128 + 64 * 8 + 4 * math.ceil(L / 128) + k * 4 for L in lengths)
+
+
+def time_events(fn, steps, warmup, torch):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i, (a, b) in enumerate(evs):
+        a.record()
+        fn(warmup + i)
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    per = [a.elapsed_time(b) for a, b in evs]            # ms, device time of the launches of one step
+    return wall, sum(per) / len(per), min(per)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
+              "(sharding over GPUs is described in DESIGN.md, not implemented)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import pypto_amd
+    from pypto_amd.synthetic import config_lengths, gen_indexer_inputs, gen_sfa_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ------------------------------------------------------------------ inputs (configuration 2)
+    B, S1, NQ, K = 32, 1, 128, 2048
+    lengths = config_lengths(2, seed=args.seed)
+    li = gen_indexer_inputs(B, S1, lengths, selected_count=K, seed=args.seed, variant="fp32")
+    sfa = gen_sfa_inputs(B, S1, NQ, lengths, topk=K, seed=args.seed + 1, block_table=li.block_table,
+                         block_num=li.block_num, topk_indices=torch.zeros([B, K], dtype=torch.int32))
+    li_d, sfa_d = li.to(dev), sfa.to(dev)
+
+    # ROT selections: the indexer run on ROT different query sets over the same key cache
+    g = torch.Generator().manual_seed(args.seed + 77)
+    sel = []
+    idx_queries = []
+    for r in range(ROT):
+        q = li.idx_query if r == 0 else torch.randint(-127, 128, li.idx_query.shape, generator=g, dtype=torch.int8)
+        qd = q.to(dev)
+        idx_queries.append(qd)
+        res = torch.empty([B, 1, K], dtype=torch.int32, device=dev)
+        pypto_amd.lightning_indexer_decode(qd, li_d.idx_query_scale, li_d.idx_key_cache, li_d.idx_key_scale,
+                                           li_d.idx_weight, li_d.act_seq_key, li_d.block_table, res, None, None, K)
+        sel.append(res.reshape(B, K).contiguous())
+    torch.cuda.synchronize()
+    out = torch.zeros([B, S1, NQ, 512], dtype=torch.bfloat16, device=dev)
+
+    def sfa_step(i):
+        pypto_amd.sparse_flash_attention_quant_d(sfa_d.query_nope, sfa_d.query_rope, sfa_d.key_nope_2d,
+                                                 sfa_d.key_rope_2d, sfa_d.k_nope_scales, sel[i % ROT],
+                                                 sfa_d.block_table, sfa_d.kv_act_seqs, out, NQ, 1,
+                                                 sfa.softmax_scale, K, 128, sfa.max_blocknum_perbatch, None)
+
+    # ------------------------------------------------------------------ timed region (attention)
+    for i in range(args.warmup):
+        sfa_step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        sfa_step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    # device-side duration of the step's launches, HIP events on the stream the kernels run on
+    _, ev_avg_ms, ev_min_ms = time_events(sfa_step, args.steps, 0, torch)
+
+    cur_seqs = [min(L, K) for L in lengths]
+    byt, flops = sfa_algorithmic_work(cur_seqs, NQ)
+    achieved_tflops = flops / (ev_avg_ms * 1e-3) / 1e12
+    achieved_gbs = byt / (ev_avg_ms * 1e-3) / 1e9
+
+    # ------------------------------------------------------------------ indexer timings
+    res = torch.empty([B, 1, K], dtype=torch.int32, device=dev)
+
+    def li_step(i):
+        pypto_amd.lightning_indexer_decode(idx_queries[i % ROT], li_d.idx_query_scale, li_d.idx_key_cache,
+                                           li_d.idx_key_scale, li_d.idx_weight, li_d.act_seq_key, li_d.block_table,
+                                           res, None, None, K)
+    _, li2_avg_ms, _ = time_events(li_step, max(args.steps // 4, 5), 3, torch)
+    li2_bytes = indexer_algorithmic_bytes(lengths, 4)
+
+    li1 = gen_indexer_inputs(4, 1, config_lengths(1), selected_count=K, seed=1, variant="fp32").to(dev)
+
+    def li1_step(i):
+        pypto_amd.lightning_indexer_decode(li1.idx_query, li1.idx_query_scale, li1.idx_key_cache, li1.idx_key_scale,
+                                           li1.idx_weight, li1.act_seq_key, li1.block_table, li1.topk_res, None, None,
+                                           K)
+    _, li1_avg_ms, _ = time_events(li1_step, max(args.steps // 4, 5), 3, torch)
+    li1_bytes = indexer_algorithmic_bytes(config_lengths(1), 4)
+
+    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import c_oracle
+        nthreads = min(c_oracle.get_threads(), os.cpu_count() or 1)
+        c_oracle.set_threads(nthreads)
+        sample_b = 4
+        idx_cpu = sel[0][:sample_b].cpu()
+        t_cpu0 = time.perf_counter()
+        c_oracle.sfa_quant(sfa.query_nope[:sample_b * NQ], sfa.query_rope[:sample_b * NQ], sfa.key_nope_2d,
+                           sfa.key_rope_2d, sfa.k_nope_scales, idx_cpu, sfa.block_table[:sample_b],
+                           sfa.kv_act_seqs[:sample_b], sample_b, 1, NQ, K, 128, sfa.softmax_scale, s2_tile=0)
+        t_cpu = time.perf_counter() - t_cpu0
+        cpu = {"value": sample_b / t_cpu, "unit": "tokens/s", "cores": nthreads, "kind": "port",
+               "sample": f"first {sample_b} of the {B} sequences of the same batch, scalar C golden with OpenMP "
+                         f"over heads, {t_cpu:.2f} s"}
+
+    line = {
+        "metric": "sfa_decode_tokens_per_s",
+        "value": B * S1 / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "configs[2]: SFA decode B=32 S_q=1 128 heads d=576/512 topk=2048 (from the indexer) "
+                               "int8 latent KV + 4 fp32 scales/token + bf16 rope, KV 8192-65536 paged bs=128, "
+                               f"shuffled block table, {ROT} rotating selections",
+                   "kv_rows": int(sfa.key_nope_2d.shape[0]), "sum_kv_len": int(sum(lengths))},
+        "roofline": {"bound": "mfma", "achieved": achieved_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved_tflops / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel": "sfa_decode_kernel<4> + sfa_combine_kernel (one step)",
+                     "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "flops_per_launch": flops},
+        "roofline_hbm": {"bound": "hbm", "achieved": achieved_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": achieved_gbs / PEAK_HBM_GBS, "bytes_per_launch": byt},
+        "indexer": {"configs[2]_us_per_step": li2_avg_ms * 1e3, "configs[2]_hbm_frac": li2_bytes / (li2_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                    "configs[1]_us_per_step": li1_avg_ms * 1e3, "configs[1]_hbm_frac": li1_bytes / (li1_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                    "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes, "scale_dtype": "fp32", "weight_dtype": "bf16"},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

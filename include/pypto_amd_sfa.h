@@ -1,0 +1,164 @@
+/*
+ * C ABI of the MI355X (gfx950) implementation of the quantized DeepSeek-V3.2
+ * sparse-attention path: the lightning indexer (score + top-k select) and the
+ * sparse flash attention that consumes its indices.
+ *
+ * Plain pointers and sizes only; every pointer is a DEVICE pointer unless stated
+ * otherwise.  The caller owns all memory, including outputs and the workspace.
+ * Launches are asynchronous on the HIP stream passed in (a hipStream_t cast to
+ * void*; NULL = the default stream); nothing here synchronises.
+ *
+ * Return value: 0 on success, a negative PTO_E_* code otherwise;
+ * pto_last_error() returns a thread-local, NUL-terminated description of the
+ * last failure on the calling thread.
+ *
+ * What each entry point replaces in the reference (paths relative to the
+ * reference tree):
+ *
+ *   pto_sfa_quant_launch
+ *       the device execution of sparse_flash_attention_quant_d / _p
+ *       (examples/models/deepseek_v32_exp/sparse_flash_attention_quant_impl.py:437-476,
+ *       499-538), i.e. what python/pypto/runtime.py:153 dispatches through
+ *       ExportedOperatorDeviceLaunchOnceWithDeviceTensorData
+ *       (framework/src/machine/runtime/device_launcher_binding.h:204-209).
+ *   pto_li_decode_launch
+ *       the device execution of lightning_indexer_decode
+ *       (examples/models/deepseek_v32_exp/lightning_indexer_quant_impl.py:315-346),
+ *       same dispatch point.
+ *   pto_*_workspace_bytes
+ *       the workspace query the reference runtime performs before a launch
+ *       (python/pypto/runtime.py:151-152, GetWorkSpaceSize).
+ */
+#ifndef PYPTO_AMD_SFA_H
+#define PYPTO_AMD_SFA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTO_OK 0
+#define PTO_E_INVALID_ARG (-1) /* NULL pointer, unsupported shape or dtype code      */
+#define PTO_E_WORKSPACE (-2)   /* workspace missing or smaller than *_workspace_bytes */
+#define PTO_E_LAUNCH (-3)      /* the HIP runtime refused the launch                  */
+#define PTO_E_NO_DEVICE (-4)   /* no gfx950 device / code object not loadable        */
+
+/* element types of the indexer's scale and weight tensors */
+#define PTO_DT_FP16 0
+#define PTO_DT_FP32 1
+#define PTO_DT_BF16 2
+
+/*
+ * Sparse flash attention over the paged int8 latent-KV cache.
+ * Tensor names, shapes and layouts are those of sparse_flash_attention_quant_d
+ * (sparse_flash_attention_quant_impl.py:45-85 in the reference example):
+ *
+ *   query_nope    [b*s1*nq, 512]            bf16
+ *   query_rope    [b*s1*nq, 64]             bf16
+ *   key_nope_2d   [kv_rows, 512]            int8    kv_rows = block_num*block_size
+ *   key_rope_2d   [kv_rows, 64]             bf16
+ *   k_nope_scales [kv_rows, 4]              fp32    one scale per 128 channels
+ *   topk_indices  [b*s1, n_kv*topk]         int32   logical key positions
+ *   block_table   [b, max_blocknum_perbatch] int32  logical block -> physical block
+ *   kv_act_seqs   [b]                        int32
+ *   attention_out [b, s1, nq, 512]          bf16    written in place
+ *
+ * Query row (bi, si) attends to the first
+ *   cur_seq = min(max(kv_act_seqs[bi] - s1 + 1 + si, 0), topk)
+ * entries of its index row; rows with cur_seq == 0 are written as zeros.
+ * Indices that would address memory outside [0, kv_rows) are clamped into it
+ * (the reference reads unchecked); their contribution is unspecified.
+ *
+ * Constraints: n_kv == 1, topk >= 1, block_size >= 1, nq >= 1.
+ * num_splits: how many workgroups share one query row's keys (0 = choose).
+ */
+typedef struct PtoSfaQuantArgs {
+    const void *query_nope;
+    const void *query_rope;
+    const void *key_nope_2d;
+    const void *key_rope_2d;
+    const void *k_nope_scales;
+    const int32_t *topk_indices;
+    const int32_t *block_table;
+    const int32_t *kv_act_seqs;
+    void *attention_out;
+    void *workspace;
+    size_t workspace_bytes;
+    int64_t b;
+    int64_t s1;
+    int64_t nq;
+    int64_t n_kv;
+    int64_t topk;
+    int64_t block_size;
+    int64_t max_blocknum_perbatch;
+    int64_t kv_rows;
+    float softmax_scale;
+    int32_t num_splits;
+} PtoSfaQuantArgs;
+
+int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *args, size_t *bytes);
+int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
+
+/*
+ * Lightning indexer, decode form (lightning_indexer_quant_impl.py:52-82 in the
+ * reference example):
+ *
+ *   idx_query       [t, n_heads, head_dim]                 int8   t = b*s1
+ *   idx_query_scale [t, n_heads]                           q_scale_dtype
+ *   idx_key_cache   [block_num, block_size, 1, head_dim]   int8
+ *   idx_key_scale   [block_num, block_size, 1]             k_scale_dtype
+ *   idx_weight      [t, n_heads]                           weight_dtype
+ *   act_seq_key     [b]                                    int32
+ *   block_table     [b, max_blocknum_perbatch]             int32
+ *   topk_res        [t, 1, selected_count]                 int32  written in place
+ *
+ * score[s, j] = (sum_h w_scale[s,h] * fp16(relu(q[s,h,:] . k[j,:]) / 2048)) * k_scale[j]
+ * with the head sum taken in fp32, h ascending, product rounded before the add;
+ * w_scale = fp16(q_scale * weight) when both are fp16, else the fp32 product.
+ * Query token s of batch bi sees positions 0 .. act_seq_key[bi] - (s1-1-s) - 1;
+ * the selected_count best are written ordered by (score descending, position
+ * ascending), padded with -1.
+ *
+ * Constraints: n_heads == 64, head_dim == 128, 1 <= selected_count <= 2048,
+ * max_blocknum_perbatch * block_size <= 131072, block_size a multiple of 32.
+ */
+typedef struct PtoLiDecodeArgs {
+    const int8_t *idx_query;
+    const void *idx_query_scale;
+    const int8_t *idx_key_cache;
+    const void *idx_key_scale;
+    const void *idx_weight;
+    const int32_t *act_seq_key;
+    const int32_t *block_table;
+    int32_t *topk_res;
+    void *workspace;
+    size_t workspace_bytes;
+    int64_t t;
+    int64_t b;
+    int64_t n_heads;
+    int64_t head_dim;
+    int64_t block_num;
+    int64_t block_size;
+    int64_t max_blocknum_perbatch;
+    int64_t selected_count;
+    int32_t q_scale_dtype;
+    int32_t k_scale_dtype;
+    int32_t weight_dtype;
+    int32_t reserved;
+} PtoLiDecodeArgs;
+
+int pto_li_decode_workspace_bytes(const PtoLiDecodeArgs *args, size_t *bytes);
+int pto_li_decode_launch(const PtoLiDecodeArgs *args, void *hip_stream);
+
+/* Thread-local description of the last error on this thread ("" if none). */
+const char *pto_last_error(void);
+
+/* Library version, "major.minor.patch". */
+const char *pto_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PYPTO_AMD_SFA_H */

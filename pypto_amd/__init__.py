@@ -1,0 +1,17 @@
+"""pypto_amd -- MI355X (gfx950) implementation of the quantized DeepSeek-V3.2 sparse-attention path.
+
+Operators (same names and signatures as the reference examples they replace):
+
+* :func:`sparse_flash_attention_quant_d` / :func:`sparse_flash_attention_quant_p`
+* :func:`lightning_indexer_decode`
+
+plus :func:`from_torch`, the tensor hand-over of the reference's jit convention.  The computation
+runs in hand-written HIP kernels behind a C ABI (``include/pypto_amd_sfa.h``); there is no CPU
+fallback.
+"""
+from .converter import Tensor, from_torch  # noqa: F401
+from .lightning_indexer_quant_impl import LightningIndexerConfigs, lightning_indexer_decode  # noqa: F401
+from .sparse_flash_attention_quant_impl import (SaTileShapeConfig, sparse_flash_attention_quant_d,  # noqa: F401
+                                                sparse_flash_attention_quant_p)
+
+__version__ = "0.1.0"

@@ -1,0 +1,229 @@
+// C ABI of the library: argument validation, workspace sizing, launch heuristics.
+// Declarations and the reference interfaces they stand in for: include/pypto_amd_sfa.h.
+#include "pypto_amd_sfa.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "li_kernels.h"
+#include "sfa_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int cu_count()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cached = n;
+        else
+            cached = 256;
+    }
+    return cached;
+}
+
+struct SfaPlan {
+    int waves;
+    int hgroups;
+    int nsplit;
+    size_t part_o_bytes;
+    size_t part_ml_bytes;
+};
+
+int sfa_check(const PtoSfaQuantArgs *a)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "sfa: args is NULL");
+    if (a->b < 1 || a->s1 < 1 || a->nq < 1) return fail(PTO_E_INVALID_ARG, "sfa: b, s1, nq must be >= 1");
+    if (a->n_kv != 1) return fail(PTO_E_INVALID_ARG, "sfa: n_kv must be 1 (got %lld)", (long long)a->n_kv);
+    if (a->topk < 1) return fail(PTO_E_INVALID_ARG, "sfa: topk must be >= 1");
+    if (a->block_size < 1 || a->max_blocknum_perbatch < 1)
+        return fail(PTO_E_INVALID_ARG, "sfa: block_size and max_blocknum_perbatch must be >= 1");
+    if (a->kv_rows < 1) return fail(PTO_E_INVALID_ARG, "sfa: kv_rows must be >= 1");
+    if (a->b * a->s1 > (1ll << 24) || a->nq > 65536 || a->topk > (1ll << 24) || a->kv_rows > 0x7fffffffll)
+        return fail(PTO_E_INVALID_ARG, "sfa: shape out of the supported range");
+    if (a->num_splits < 0) return fail(PTO_E_INVALID_ARG, "sfa: num_splits must be >= 0");
+    if (!std::isfinite(a->softmax_scale)) return fail(PTO_E_INVALID_ARG, "sfa: softmax_scale is not finite");
+    return PTO_OK;
+}
+
+SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
+{
+    SfaPlan pl;
+    pl.waves = a->nq > 64 ? 4 : (a->nq > 32 ? 2 : 1);
+    const int heads_per_wg = 32 * pl.waves;
+    pl.hgroups = (int)((a->nq + heads_per_wg - 1) / heads_per_wg);
+    const long long rows = a->b * a->s1;
+    const int tiles = (int)((a->topk + pto::SFA_KEY_TILE - 1) / pto::SFA_KEY_TILE);
+    const int min_split = (int)((a->topk + pto::SFA_MAX_CHUNK - 1) / pto::SFA_MAX_CHUNK);
+    int ns = a->num_splits;
+    if (ns == 0) {
+        // fill the chip once; a split shorter than four tiles is all prologue
+        const long long wgs = rows * pl.hgroups;
+        ns = (int)((cu_count() + wgs - 1) / wgs);
+        const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
+        ns = ns > max_split ? max_split : ns;
+    }
+    ns = ns < min_split ? min_split : ns;
+    ns = ns > tiles ? tiles : ns;
+    ns = ns < 1 ? 1 : ns;
+    pl.nsplit = ns;
+    if (ns > 1) {
+        pl.part_o_bytes = (size_t)rows * ns * a->nq * 512 * sizeof(float);
+        pl.part_ml_bytes = (size_t)rows * ns * a->nq * 2 * sizeof(float);
+    } else {
+        pl.part_o_bytes = pl.part_ml_bytes = 0;
+    }
+    return pl;
+}
+
+int li_check(const PtoLiDecodeArgs *a)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "li: args is NULL");
+    if (a->t < 1 || a->b < 1 || a->t % a->b != 0) return fail(PTO_E_INVALID_ARG, "li: t must be a positive multiple of b");
+    if (a->n_heads != 64 || a->head_dim != 128)
+        return fail(PTO_E_INVALID_ARG, "li: n_heads must be 64 and head_dim 128 (got %lld, %lld)", (long long)a->n_heads,
+                    (long long)a->head_dim);
+    if (a->selected_count < 1 || a->selected_count > pto::LI_MAX_SELECT)
+        return fail(PTO_E_INVALID_ARG, "li: selected_count must be in [1, %d]", pto::LI_MAX_SELECT);
+    if (a->block_size < 32 || a->block_size % 32 != 0) return fail(PTO_E_INVALID_ARG, "li: block_size must be a multiple of 32");
+    if (a->block_num < 1 || a->max_blocknum_perbatch < 1) return fail(PTO_E_INVALID_ARG, "li: block_num and max_blocknum_perbatch must be >= 1");
+    if (a->max_blocknum_perbatch * a->block_size > pto::LI_MAX_SEQ)
+        return fail(PTO_E_INVALID_ARG, "li: max_blocknum_perbatch * block_size exceeds %d", pto::LI_MAX_SEQ);
+    if (a->t > (1ll << 20) || a->block_num * a->block_size > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "li: shape out of the supported range");
+    const int dts[3] = {a->q_scale_dtype, a->k_scale_dtype, a->weight_dtype};
+    for (int d : dts)
+        if (d != PTO_DT_FP16 && d != PTO_DT_FP32 && d != PTO_DT_BF16) return fail(PTO_E_INVALID_ARG, "li: unknown dtype code %d", d);
+    return PTO_OK;
+}
+
+size_t li_ws_bytes(const PtoLiDecodeArgs *a)
+{
+    // score rows [t, max_blocknum_perbatch*block_size] fp32 + w_scale [t, 64] fp32
+    const size_t stride = (size_t)a->max_blocknum_perbatch * a->block_size;
+    return (size_t)a->t * stride * sizeof(float) + (size_t)a->t * 64 * sizeof(float);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *pto_last_error(void) { return g_err; }
+
+const char *pto_version(void) { return "0.1.0"; }
+
+int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
+{
+    if (!bytes) return fail(PTO_E_INVALID_ARG, "sfa: bytes is NULL");
+    int rc = sfa_check(a);
+    if (rc != PTO_OK) return rc;
+    const SfaPlan pl = sfa_plan(a);
+    *bytes = pl.part_o_bytes + pl.part_ml_bytes;
+    return PTO_OK;
+}
+
+int pto_sfa_quant_launch(const PtoSfaQuantArgs *a, void *hip_stream)
+{
+    int rc = sfa_check(a);
+    if (rc != PTO_OK) return rc;
+    if (!a->query_nope || !a->query_rope || !a->key_nope_2d || !a->key_rope_2d || !a->k_nope_scales || !a->topk_indices ||
+        !a->block_table || !a->kv_act_seqs || !a->attention_out)
+        return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
+    const SfaPlan pl = sfa_plan(a);
+    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
+    if (need > 0 && (!a->workspace || a->workspace_bytes < need))
+        return fail(PTO_E_WORKSPACE, "sfa: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+
+    pto::SfaParams p;
+    p.q_nope = static_cast<const uint16_t *>(a->query_nope);
+    p.q_rope = static_cast<const uint16_t *>(a->query_rope);
+    p.kn = static_cast<const int8_t *>(a->key_nope_2d);
+    p.kr = static_cast<const uint16_t *>(a->key_rope_2d);
+    p.ksc = static_cast<const float *>(a->k_nope_scales);
+    p.topk_idx = a->topk_indices;
+    p.bt = a->block_table;
+    p.act = a->kv_act_seqs;
+    p.out = static_cast<uint16_t *>(a->attention_out);
+    p.part_o = static_cast<float *>(a->workspace);
+    p.part_ml = need > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
+    p.kv_rows = a->kv_rows;
+    p.T = (int)(a->b * a->s1);
+    p.S1 = (int)a->s1;
+    p.NQ = (int)a->nq;
+    p.topk = (int)a->topk;
+    p.bs = (int)a->block_size;
+    p.maxblk = (int)a->max_blocknum_perbatch;
+    p.nsplit = pl.nsplit;
+    p.hgroups = pl.hgroups;
+    p.waves = pl.waves;
+    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    hipError_t e = pto::sfa_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "sfa: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
+int pto_li_decode_workspace_bytes(const PtoLiDecodeArgs *a, size_t *bytes)
+{
+    if (!bytes) return fail(PTO_E_INVALID_ARG, "li: bytes is NULL");
+    int rc = li_check(a);
+    if (rc != PTO_OK) return rc;
+    *bytes = li_ws_bytes(a);
+    return PTO_OK;
+}
+
+int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
+{
+    int rc = li_check(a);
+    if (rc != PTO_OK) return rc;
+    if (!a->idx_query || !a->idx_query_scale || !a->idx_key_cache || !a->idx_key_scale || !a->idx_weight || !a->act_seq_key ||
+        !a->block_table || !a->topk_res)
+        return fail(PTO_E_INVALID_ARG, "li: a tensor pointer is NULL");
+    const size_t need = li_ws_bytes(a);
+    if (!a->workspace || a->workspace_bytes < need)
+        return fail(PTO_E_WORKSPACE, "li: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+
+    pto::LiParams p;
+    p.q = a->idx_query;
+    p.q_scale = a->idx_query_scale;
+    p.kcache = a->idx_key_cache;
+    p.k_scale = a->idx_key_scale;
+    p.weight = a->idx_weight;
+    p.act = a->act_seq_key;
+    p.bt = a->block_table;
+    p.topk_res = a->topk_res;
+    p.T = (int)a->t;
+    p.B = (int)a->b;
+    p.S1 = (int)(a->t / a->b);
+    p.bs = (int)a->block_size;
+    p.maxblk = (int)a->max_blocknum_perbatch;
+    p.nblocks = (int)a->block_num;
+    p.k = (int)a->selected_count;
+    p.score_stride = (long long)a->max_blocknum_perbatch * a->block_size;
+    p.scores = static_cast<float *>(a->workspace);
+    p.w_scale = p.scores + (size_t)a->t * p.score_stride;
+    p.q_dt = a->q_scale_dtype;
+    p.k_dt = a->k_scale_dtype;
+    p.w_dt = a->weight_dtype;
+    p.num_cu = cu_count();
+    hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,32 @@
+// Launch parameters of the lightning-indexer kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+constexpr int LI_MAX_SELECT = 2048;     // most indices one query token can receive
+constexpr int LI_MAX_SEQ = 128 * 1024;  // longest key sequence
+constexpr int LI_HEADS = 64;
+constexpr int LI_DIM = 128;
+
+struct LiParams {
+    const int8_t *q;        // [T, 64, 128]
+    const void *q_scale;    // [T, 64]    q_dt
+    const int8_t *kcache;   // [nblocks*bs, 128]
+    const void *k_scale;    // [nblocks*bs]  k_dt
+    const void *weight;     // [T, 64]    w_dt
+    const int32_t *act;     // [B]
+    const int32_t *bt;      // [B, maxblk]
+    int32_t *topk_res;      // [T, k]
+    float *scores;          // workspace [T, score_stride]
+    float *w_scale;         // workspace [T, 64]
+    long long score_stride;
+    int T, B, S1, bs, maxblk, nblocks, k;
+    int q_dt, k_dt, w_dt;   // PTO_DT_* codes
+    int num_cu;
+};
+
+hipError_t li_launch(const LiParams &p, hipStream_t stream);
+
+}  // namespace pto

@@ -1,0 +1,144 @@
+// pybind11 face of the C ABI.  Tensors cross as raw device addresses (torch's data_ptr()) and the
+// HIP stream as an integer handle; no torch types appear here.  Argument errors raise ValueError,
+// everything else RuntimeError, carrying the library's own message.
+#include <pybind11/pybind11.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "pypto_amd_sfa.h"
+
+namespace py = pybind11;
+
+namespace {
+
+void check(int rc)
+{
+    if (rc == PTO_OK) return;
+    const std::string msg = pto_last_error();
+    if (rc == PTO_E_INVALID_ARG) throw py::value_error(msg);
+    throw std::runtime_error(msg);
+}
+
+template <typename T> T *ptr(std::uintptr_t v) { return reinterpret_cast<T *>(v); }
+
+PtoSfaQuantArgs sfa_args(std::uintptr_t query_nope, std::uintptr_t query_rope, std::uintptr_t key_nope_2d,
+                         std::uintptr_t key_rope_2d, std::uintptr_t k_nope_scales, std::uintptr_t topk_indices,
+                         std::uintptr_t block_table, std::uintptr_t kv_act_seqs, std::uintptr_t attention_out,
+                         std::uintptr_t workspace, size_t workspace_bytes, int64_t b, int64_t s1, int64_t nq,
+                         int64_t n_kv, int64_t topk, int64_t block_size, int64_t max_blocknum_perbatch,
+                         int64_t kv_rows, double softmax_scale, int num_splits)
+{
+    PtoSfaQuantArgs a{};
+    a.query_nope = ptr<const void>(query_nope);
+    a.query_rope = ptr<const void>(query_rope);
+    a.key_nope_2d = ptr<const void>(key_nope_2d);
+    a.key_rope_2d = ptr<const void>(key_rope_2d);
+    a.k_nope_scales = ptr<const void>(k_nope_scales);
+    a.topk_indices = ptr<const int32_t>(topk_indices);
+    a.block_table = ptr<const int32_t>(block_table);
+    a.kv_act_seqs = ptr<const int32_t>(kv_act_seqs);
+    a.attention_out = ptr<void>(attention_out);
+    a.workspace = ptr<void>(workspace);
+    a.workspace_bytes = workspace_bytes;
+    a.b = b;
+    a.s1 = s1;
+    a.nq = nq;
+    a.n_kv = n_kv;
+    a.topk = topk;
+    a.block_size = block_size;
+    a.max_blocknum_perbatch = max_blocknum_perbatch;
+    a.kv_rows = kv_rows;
+    a.softmax_scale = static_cast<float>(softmax_scale);
+    a.num_splits = num_splits;
+    return a;
+}
+
+PtoLiDecodeArgs li_args(std::uintptr_t idx_query, std::uintptr_t idx_query_scale, std::uintptr_t idx_key_cache,
+                        std::uintptr_t idx_key_scale, std::uintptr_t idx_weight, std::uintptr_t act_seq_key,
+                        std::uintptr_t block_table, std::uintptr_t topk_res, std::uintptr_t workspace,
+                        size_t workspace_bytes, int64_t t, int64_t b, int64_t n_heads, int64_t head_dim,
+                        int64_t block_num, int64_t block_size, int64_t max_blocknum_perbatch, int64_t selected_count,
+                        int q_scale_dtype, int k_scale_dtype, int weight_dtype)
+{
+    PtoLiDecodeArgs a{};
+    a.idx_query = ptr<const int8_t>(idx_query);
+    a.idx_query_scale = ptr<const void>(idx_query_scale);
+    a.idx_key_cache = ptr<const int8_t>(idx_key_cache);
+    a.idx_key_scale = ptr<const void>(idx_key_scale);
+    a.idx_weight = ptr<const void>(idx_weight);
+    a.act_seq_key = ptr<const int32_t>(act_seq_key);
+    a.block_table = ptr<const int32_t>(block_table);
+    a.topk_res = ptr<int32_t>(topk_res);
+    a.workspace = ptr<void>(workspace);
+    a.workspace_bytes = workspace_bytes;
+    a.t = t;
+    a.b = b;
+    a.n_heads = n_heads;
+    a.head_dim = head_dim;
+    a.block_num = block_num;
+    a.block_size = block_size;
+    a.max_blocknum_perbatch = max_blocknum_perbatch;
+    a.selected_count = selected_count;
+    a.q_scale_dtype = q_scale_dtype;
+    a.k_scale_dtype = k_scale_dtype;
+    a.weight_dtype = weight_dtype;
+    return a;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(_C, m)
+{
+    m.doc() = "MI355X sparse flash attention + lightning indexer (C ABI: include/pypto_amd_sfa.h)";
+    m.attr("DT_FP16") = PTO_DT_FP16;
+    m.attr("DT_FP32") = PTO_DT_FP32;
+    m.attr("DT_BF16") = PTO_DT_BF16;
+    m.def("version", []() { return std::string(pto_version()); });
+
+    m.def("sfa_quant_workspace_bytes",
+          [](int64_t b, int64_t s1, int64_t nq, int64_t n_kv, int64_t topk, int64_t block_size,
+             int64_t max_blocknum_perbatch, int64_t kv_rows, double softmax_scale, int num_splits) {
+              PtoSfaQuantArgs a = sfa_args(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, b, s1, nq, n_kv, topk, block_size,
+                                           max_blocknum_perbatch, kv_rows, softmax_scale, num_splits);
+              size_t bytes = 0;
+              check(pto_sfa_quant_workspace_bytes(&a, &bytes));
+              return bytes;
+          });
+    m.def("sfa_quant_launch",
+          [](std::uintptr_t query_nope, std::uintptr_t query_rope, std::uintptr_t key_nope_2d, std::uintptr_t key_rope_2d,
+             std::uintptr_t k_nope_scales, std::uintptr_t topk_indices, std::uintptr_t block_table,
+             std::uintptr_t kv_act_seqs, std::uintptr_t attention_out, std::uintptr_t workspace, size_t workspace_bytes,
+             int64_t b, int64_t s1, int64_t nq, int64_t n_kv, int64_t topk, int64_t block_size,
+             int64_t max_blocknum_perbatch, int64_t kv_rows, double softmax_scale, int num_splits,
+             std::uintptr_t stream) {
+              PtoSfaQuantArgs a = sfa_args(query_nope, query_rope, key_nope_2d, key_rope_2d, k_nope_scales, topk_indices,
+                                           block_table, kv_act_seqs, attention_out, workspace, workspace_bytes, b, s1, nq,
+                                           n_kv, topk, block_size, max_blocknum_perbatch, kv_rows, softmax_scale,
+                                           num_splits);
+              check(pto_sfa_quant_launch(&a, ptr<void>(stream)));
+          });
+
+    m.def("li_decode_workspace_bytes",
+          [](int64_t t, int64_t b, int64_t n_heads, int64_t head_dim, int64_t block_num, int64_t block_size,
+             int64_t max_blocknum_perbatch, int64_t selected_count, int q_dt, int k_dt, int w_dt) {
+              PtoLiDecodeArgs a = li_args(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, t, b, n_heads, head_dim, block_num, block_size,
+                                          max_blocknum_perbatch, selected_count, q_dt, k_dt, w_dt);
+              size_t bytes = 0;
+              check(pto_li_decode_workspace_bytes(&a, &bytes));
+              return bytes;
+          });
+    m.def("li_decode_launch",
+          [](std::uintptr_t idx_query, std::uintptr_t idx_query_scale, std::uintptr_t idx_key_cache,
+             std::uintptr_t idx_key_scale, std::uintptr_t idx_weight, std::uintptr_t act_seq_key,
+             std::uintptr_t block_table, std::uintptr_t topk_res, std::uintptr_t workspace, size_t workspace_bytes,
+             int64_t t, int64_t b, int64_t n_heads, int64_t head_dim, int64_t block_num, int64_t block_size,
+             int64_t max_blocknum_perbatch, int64_t selected_count, int q_dt, int k_dt, int w_dt,
+             std::uintptr_t stream) {
+              PtoLiDecodeArgs a = li_args(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight, act_seq_key,
+                                          block_table, topk_res, workspace, workspace_bytes, t, b, n_heads, head_dim,
+                                          block_num, block_size, max_blocknum_perbatch, selected_count, q_dt, k_dt, w_dt);
+              check(pto_li_decode_launch(&a, ptr<void>(stream)));
+          });
+}

@@ -1,0 +1,33 @@
+// Launch parameters of the sparse-flash-attention kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+constexpr int SFA_MAX_CHUNK = 2048;   // most keys one workgroup handles (row-translation table in LDS)
+constexpr int SFA_KEY_TILE = 32;
+
+struct SfaParams {
+    const uint16_t *q_nope;   // [T*NQ, 512] bf16
+    const uint16_t *q_rope;   // [T*NQ, 64]  bf16
+    const int8_t *kn;         // [kv_rows, 512]
+    const uint16_t *kr;       // [kv_rows, 64] bf16
+    const float *ksc;         // [kv_rows, 4]
+    const int32_t *topk_idx;  // [T, topk]
+    const int32_t *bt;        // [B, maxblk]
+    const int32_t *act;       // [B]
+    uint16_t *out;            // [T*NQ, 512] bf16
+    float *part_o;            // [T, nsplit, NQ, 512] un-normalised partial sums (nsplit > 1)
+    float *part_ml;           // [T, nsplit, NQ, 2]   running max (log2 domain) and row sum
+    long long kv_rows;
+    int T, S1, NQ, topk, bs, maxblk;
+    int nsplit;               // key splits per query row
+    int hgroups;              // head groups per query row (32*waves heads each)
+    int waves;                // waves per workgroup: 1, 2 or 4
+    float scale_log2;         // softmax_scale * log2(e)
+};
+
+hipError_t sfa_launch(const SfaParams &p, hipStream_t stream);
+
+}  // namespace pto

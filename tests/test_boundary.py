@@ -1,0 +1,87 @@
+"""The C-ABI library loads and exports every symbol the header declares; host-side argument
+checking of the C ABI and of the Python operators (no GPU needed: nothing is launched)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "pypto_amd", "libpypto_amd_sfa.so")
+HEADER = os.path.join(ROOT, "include", "pypto_amd_sfa.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        from pypto_amd.build import build_all
+        build_all()
+    return ctypes.CDLL(LIB)
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pto_\w+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(lib):
+    names = _declared()
+    assert {"pto_sfa_quant_launch", "pto_sfa_quant_workspace_bytes", "pto_li_decode_launch",
+            "pto_li_decode_workspace_bytes", "pto_last_error", "pto_version"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_version_and_error_string(lib):
+    lib.pto_version.restype = ctypes.c_char_p
+    lib.pto_last_error.restype = ctypes.c_char_p
+    assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.pto_version())
+    n = ctypes.c_size_t(0)
+    assert lib.pto_sfa_quant_workspace_bytes(None, ctypes.byref(n)) == -1
+    assert b"NULL" in lib.pto_last_error()
+
+
+def test_pybind_workspace_and_argument_errors():
+    from pypto_amd import _native
+    C = _native.load()
+    # 32 rows x 8 splits x 128 heads x (512 + 2) floats
+    assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 20, 0.04, 8) == 32 * 8 * 128 * 514 * 4
+    assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 0      # no split needed
+    assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * 32768 * 4 + 4 * 64 * 4
+    with pytest.raises(ValueError):
+        C.sfa_quant_workspace_bytes(1, 1, 128, 2, 2048, 128, 32, 4096, 0.04, 0)      # n_kv != 1
+    with pytest.raises(ValueError):
+        C.li_decode_workspace_bytes(4, 4, 32, 128, 1024, 128, 256, 2048, 0, 0, 0)    # 32 heads
+    with pytest.raises(ValueError):
+        C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 4096, 0, 0, 0)    # selected_count > 2048
+    with pytest.raises(ValueError):
+        C.li_decode_workspace_bytes(4, 4, 64, 128, 4096, 128, 2048, 2048, 0, 0, 0)   # longer than 128K
+    with pytest.raises(ValueError):                                                  # NULL tensors
+        C.sfa_quant_launch(0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 1, 16, 1, 256, 128, 32, 4096, 0.04, 0, 0)
+
+
+def test_from_torch_contract():
+    import pypto_amd
+    t = torch.zeros(4, 6)
+    h = pypto_amd.from_torch(t, name="x", dynamic_axis=[0])
+    assert h.shape == [4, 6] and h.dtype == torch.float32 and h.data_ptr == t.data_ptr() and h.name == "x"
+    with pytest.raises(TypeError):
+        pypto_amd.from_torch([1, 2, 3])
+    with pytest.raises(RuntimeError):
+        pypto_amd.from_torch(t.t())
+
+
+def test_operators_refuse_cpu_tensors_loudly():
+    """There is no CPU fallback behind the operator names."""
+    import pypto_amd
+    from pypto_amd.synthetic import gen_sfa_inputs, gen_indexer_inputs
+    inp = gen_sfa_inputs(1, 1, 16, [256], topk=64, seed=0)
+    out = torch.zeros(1, 1, 16, 512, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        pypto_amd.sparse_flash_attention_quant_d(*inp.operator_tensors(), out, 16, 1, inp.softmax_scale, 64, 128,
+                                                 inp.max_blocknum_perbatch, None)
+    li = gen_indexer_inputs(1, 1, [256], selected_count=64, seed=0)
+    with pytest.raises(RuntimeError):
+        pypto_amd.lightning_indexer_decode(*li.operator_tensors(), None, None, 64)

@@ -1,0 +1,81 @@
+"""Parity of the HIP lightning indexer (through the operator, pybind11 and the C ABI) against the CPU
+oracle.  The bar is bit-exact indices."""
+import numpy as np
+import pytest
+import torch
+
+import pypto_amd
+from pypto_amd.synthetic import gen_indexer_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def run_op(inp):
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    d.topk_res.fill_(-7)
+    ts = [pypto_amd.from_torch(t) for t in d.operator_tensors()]
+    ret = pypto_amd.lightning_indexer_decode(*ts, [128, 64, 32, 16, 8, 4, 1], pypto_amd.LightningIndexerConfigs(),
+                                             inp.selected_count)
+    assert ret is None
+    torch.cuda.synchronize()
+    return d.topk_res.cpu()
+
+
+def oracle(inp, c_oracle):
+    return c_oracle.li_decode(inp.idx_query, inp.idx_query_scale, inp.idx_key_cache, inp.idx_key_scale,
+                              inp.idx_weight, inp.act_seq_key, inp.block_table, inp.selected_count)
+
+
+def assert_exact(got, ref, what):
+    if not torch.equal(got, ref):
+        bad = (got != ref).reshape(got.shape[0], -1)
+        rows = torch.nonzero(bad.any(dim=1)).reshape(-1).tolist()
+        r = rows[0]
+        cols = torch.nonzero(bad[r]).reshape(-1)[:8].tolist()
+        raise AssertionError(f"{what}: {int(bad.sum())} index mismatches in rows {rows[:8]}; row {r} cols {cols}: "
+                             f"got {got[r, 0, cols].tolist()} want {ref[r, 0, cols].tolist()}")
+
+
+@pytest.mark.parametrize("variant", ["fp16", "fp32"])
+@pytest.mark.parametrize("b,s1,act,k", [
+    (2, 1, [4096, 3000], 2048),        # above the select threshold, one ragged
+    (3, 2, [300, 129, 5], 64),         # two query tokens per sequence, causal effective lengths
+    (2, 1, [2048, 2049], 2048),        # exactly k and k+1 candidates
+    (2, 1, [100, 1], 2048),            # fewer candidates than k: padded with -1
+    (1, 4, [9000], 2048),              # s1 = 4
+    (1, 1, [33], 16),                  # partial 32-key block
+])
+def test_indexer_bit_exact(c_oracle, variant, b, s1, act, k):
+    inp = gen_indexer_inputs(b, s1, act, selected_count=k, seed=7 * b + s1 + k, variant=variant)
+    assert_exact(run_op(inp), oracle(inp, c_oracle), f"{variant} b={b} s1={s1} act={act} k={k}")
+
+
+def test_engineered_ties_and_zero_scores(c_oracle):
+    """Many equal scores: zero weights make every score +-0, duplicated key rows make exact ties."""
+    inp = gen_indexer_inputs(2, 1, [5000, 6000], selected_count=2048, seed=31, variant="fp16")
+    inp.idx_weight[0] = 0                                # token 0: all scores are zero -> positions 0..2047
+    kc = inp.idx_key_cache.reshape(-1, 128)
+    ks = inp.idx_key_scale.reshape(-1)
+    # token 1: every logical position p >= 3000 repeats the row of position p - 3000
+    pos = torch.arange(6000)
+    phys = inp.block_table[1].long()[pos // 128] * 128 + pos % 128
+    kc[phys[3000:]] = kc[phys[:3000]]
+    ks[phys[3000:]] = ks[phys[:3000]]
+    got = run_op(inp)
+    ref = oracle(inp, c_oracle)
+    assert ref[0, 0].tolist() == list(range(2048))
+    assert_exact(got, ref, "ties")
+
+
+def test_negative_weights_and_mixed_signs(c_oracle):
+    inp = gen_indexer_inputs(1, 1, [7000], selected_count=2048, seed=41, variant="fp32")
+    inp.idx_weight[:] = -inp.idx_weight.abs()            # all scores <= 0: the best are the zeros
+    assert_exact(run_op(inp), oracle(inp, c_oracle), "negative")
+
+
+def test_config1_full_size(c_oracle):
+    """B=4, KV 32768 each, shuffled block table, top-2048."""
+    for variant in ("fp16", "fp32"):
+        inp = gen_indexer_inputs(4, 1, [32768] * 4, selected_count=2048, seed=1, variant=variant)
+        assert_exact(run_op(inp), oracle(inp, c_oracle), f"cfg1 {variant}")
