@@ -85,7 +85,7 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
     ns = ns < 1 ? 1 : ns;
     pl.nsplit = ns;
     if (ns > 1) {
-        pl.part_o_bytes = (size_t)rows * ns * a->nq * 512 * sizeof(float);
+        pl.part_o_bytes = (size_t)rows * ns * a->nq * 512 * sizeof(uint16_t);
         pl.part_ml_bytes = (size_t)rows * ns * a->nq * 2 * sizeof(float);
     } else {
         pl.part_o_bytes = pl.part_ml_bytes = 0;
@@ -160,7 +160,7 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *a, void *hip_stream)
     p.bt = a->block_table;
     p.act = a->kv_act_seqs;
     p.out = static_cast<uint16_t *>(a->attention_out);
-    p.part_o = static_cast<float *>(a->workspace);
+    p.part_o = static_cast<uint16_t *>(a->workspace);
     p.part_ml = need > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
     p.kv_rows = a->kv_rows;
     p.T = (int)(a->b * a->s1);

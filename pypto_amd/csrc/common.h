@@ -9,6 +9,8 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -23,6 +25,14 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 {
     f32x2 v = {lo, hi};
     bf16x2 r = __builtin_convertvector(v, bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// two fp32 -> packed fp16 pair, round-to-nearest-even (v_cvt_pk_f16_f32)
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
+{
+    f32x2 v = {lo, hi};
+    f16x2 r = __builtin_convertvector(v, f16x2);
     return __builtin_bit_cast(uint32_t, r);
 }
 

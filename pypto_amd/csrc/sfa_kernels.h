@@ -18,8 +18,8 @@ struct SfaParams {
     const int32_t *bt;        // [B, maxblk]
     const int32_t *act;       // [B]
     uint16_t *out;            // [T*NQ, 512] bf16
-    float *part_o;            // [T, nsplit, NQ, 512] un-normalised partial sums (nsplit > 1)
-    float *part_ml;           // [T, nsplit, NQ, 2]   running max (log2 domain) and row sum
+    uint16_t *part_o;         // [T, nsplit, NQ, 512] fp16: O / l of each key split (nsplit > 1)
+    float *part_ml;           // [T, nsplit, NQ, 2]   reference max (log2 domain) and row sum of the split
     long long kv_rows;
     int T, S1, NQ, topk, bs, maxblk;
     int nsplit;               // key splits per query row

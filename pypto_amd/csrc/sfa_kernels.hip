@@ -19,6 +19,8 @@
 // the transposed V read uses the same key order, so no cross-lane movement is needed).
 // All NW waves gather and de-quantise the tile cooperatively: each selected row is read once per
 // workgroup (512 B int8 + 128 B rope + 16 B scales) and written to LDS as 576 bf16.
+#include <type_traits>
+
 #include "common.h"
 #include "sfa_kernels.h"
 
@@ -33,17 +35,21 @@ constexpr int PITCH = D + 8;      // LDS row pitch in bf16 elements (1168 B: row
 constexpr int KSTEPS = D / 16;    // 36 contraction steps of 16
 constexpr int DVB = DN / 32;      // 16 output blocks of 32 value channels
 
-// 16 int8 (one 16-byte load) times one scale -> 16 bf16 as two 16-byte LDS stores
+// 16 int8 (one 16-byte load) times one scale -> 16 bf16 as two 16-byte LDS stores.
+// x*sc is formed as fma(float(x + 128), sc, -128*sc): the byte is biased to unsigned so that a single
+// v_cvt_f32_ubyteN converts it, and the fused multiply-add rounds the exact product (x*sc) once, which
+// is bit-identical to the rounded multiply (128*sc is exact).
 __device__ __forceinline__ void dequant16(const i32x4 raw, const float sc, uint16_t *dst)
 {
+    const float bias = -128.0f * sc;
     u32x4 lo, hi;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-        const int v = raw[w];
-        const float f0 = (float)((v << 24) >> 24) * sc;
-        const float f1 = (float)((v << 16) >> 24) * sc;
-        const float f2 = (float)((v << 8) >> 24) * sc;
-        const float f3 = (float)(v >> 24) * sc;
+        const uint32_t v = (uint32_t)raw[w] ^ 0x80808080u;
+        const float f0 = __builtin_fmaf((float)(v & 0xffu), sc, bias);
+        const float f1 = __builtin_fmaf((float)((v >> 8) & 0xffu), sc, bias);
+        const float f2 = __builtin_fmaf((float)((v >> 16) & 0xffu), sc, bias);
+        const float f3 = __builtin_fmaf((float)(v >> 24), sc, bias);
         const uint32_t p0 = pack_bf16x2(f0, f1);
         const uint32_t p1 = pack_bf16x2(f2, f3);
         if (w < 2) { lo[2 * w] = p0; lo[2 * w + 1] = p1; }
@@ -78,19 +84,9 @@ __device__ __forceinline__ void acc_scale(f32x16 &acc, const float alpha)
 
 template <int I, int N> struct AccLoop {
     static __device__ __forceinline__ void scale(f32x16 *o, float a) { acc_scale(o[I], a); AccLoop<I + 1, N>::scale(o, a); }
-    static __device__ __forceinline__ void pv(f32x16 *o, const uint16_t *v, const bf16x8 pf)
-    {
-        const s16x4 lo = lds_read_tr16(v + 32 * I);
-        const s16x4 hi = lds_read_tr16(v + 32 * I + 8 * PITCH);
-        const s16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        acc_mfma(o[I], __builtin_bit_cast(bf16x8, a), pf);
-        if ((I & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // bound how many V^T reads are hoisted
-        AccLoop<I + 1, N>::pv(o, v, pf);
-    }
 };
 template <int N> struct AccLoop<N, N> {
     static __device__ __forceinline__ void scale(f32x16 *, float) {}
-    static __device__ __forceinline__ void pv(f32x16 *, const uint16_t *, const bf16x8) {}
 };
 
 // Wait states the hardware does not interlock: a matrix-core write followed by a vector-ALU read of
@@ -103,8 +99,15 @@ constexpr float RESCALE_TAU = 8.0f;   // log2 units: the reference max moves onl
 template <int NW>
 __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t tile[KT * PITCH];
+    // One LDS pool.  Prologue: all 32*NW query heads staged at once (PITCH elements each).  Loop: tile
+    // buffers of KT rows -- while tile n is consumed from one, tile n+1 (loaded into registers before
+    // the matrix products of tile n were issued) is de-quantised into the other; one barrier per tile.
+    // Epilogue: per-wave transposition slices.
+    constexpr int POOL_ROWS = 32 * NW > 2 * KT ? 32 * NW : 2 * KT;     // at least the two tile buffers
+    __shared__ __attribute__((aligned(16))) uint16_t pool[POOL_ROWS * PITCH];
     __shared__ int rows_lds[SFA_MAX_CHUNK];
+    uint16_t *const tile0 = pool;
+    uint16_t *const tile1 = pool + KT * PITCH;
 
     const int tid = threadIdx.x;
     const int w = tid >> 6;
@@ -135,27 +138,55 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     const int head = hg * (32 * NW) + w * 32 + col;
     const bool head_ok = head < p.NQ;
 
-    // logical position -> physical cache row for this split's keys
-    for (int i = tid; i < k_end - k_begin; i += NW * 64) {
-        const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + i];
-        int blk = idx / p.bs;
-        blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
-        long long row = (long long)p.bt[(size_t)b * p.maxblk + blk] * p.bs + (idx - (idx / p.bs) * p.bs);
-        row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
-        rows_lds[i] = (int)row;
-    }
-
-    // Q^T fragments: lane (head, half) holds q[head][16*ks + 8*half .. +8]; lanes of heads past NQ
-    // compute on row 0 of the query and are never stored
+    // Q^T fragments: lane (head, half) holds q[head][16*ks + 8*half .. +8].  Read straight from global
+    // memory each such load touches 32 rows; instead the workgroup's heads are copied with coalesced
+    // 16-byte loads (all issued before the first is consumed) into the LDS pool, 1168 bytes per head,
+    // and every wave picks its fragments from there.  Heads past NQ read the last head and are never
+    // stored.
     bf16x8 qf[KSTEPS];
     {
-        const size_t qrow = (size_t)t * p.NQ + (head_ok ? head : 0);
-        const uint16_t *qn = p.q_nope + qrow * DN + 8 * half;
-        const uint16_t *qr = p.q_rope + qrow * DR + 8 * half;
+        constexpr int CHUNKS = D / 8;                         // 72 16-byte chunks per head
+        constexpr int HEADS_WG = 32 * NW;
+        constexpr int ITERS = (HEADS_WG * CHUNKS) / (NW * 64);   // 36
+        u32x4 qtmp[ITERS];
 #pragma unroll
-        for (int ks = 0; ks < DN / 16; ++ks) qf[ks] = *reinterpret_cast<const bf16x8 *>(qn + 16 * ks);
+        for (int i = 0; i < ITERS; ++i) {
+            const int c = tid + i * NW * 64;
+            const int hl = c / CHUNKS;
+            const int part = c - hl * CHUNKS;
+            int hd = hg * HEADS_WG + hl;
+            hd = hd < p.NQ ? hd : p.NQ - 1;
+            const size_t qrow = (size_t)t * p.NQ + hd;
+            const uint16_t *src = part < DN / 8 ? p.q_nope + qrow * DN + 8 * part : p.q_rope + qrow * DR + 8 * (part - DN / 8);
+            qtmp[i] = *reinterpret_cast<const u32x4 *>(src);
+        }
 #pragma unroll
-        for (int ks = 0; ks < DR / 16; ++ks) qf[DN / 16 + ks] = *reinterpret_cast<const bf16x8 *>(qr + 16 * ks);
+        for (int i = 0; i < ITERS; ++i) {
+            const int c = tid + i * NW * 64;
+            const int hl = c / CHUNKS;
+            *reinterpret_cast<u32x4 *>(pool + hl * PITCH + 8 * (c - hl * CHUNKS)) = qtmp[i];
+        }
+        __syncthreads();
+        const uint16_t *qrow = pool + (w * 32 + col) * PITCH + 8 * half;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) qf[ks] = *reinterpret_cast<const bf16x8 *>(qrow + 16 * ks);
+        __syncthreads();                                      // the pool is free again
+    }
+
+    // logical position -> physical cache row for this split's keys.  The table is padded to a whole
+    // number of tiles with the row of the split's first key: keys past k_end are then loaded like any
+    // other (finite data) and masked out of the softmax, so the loop needs no per-key branches.
+    {
+        const int n_valid = k_end - k_begin;
+        const int n_pad = (n_valid + KT - 1) / KT * KT;
+        for (int i = tid; i < n_pad; i += NW * 64) {
+            const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
+            int blk = idx / p.bs;
+            blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
+            long long row = (long long)p.bt[(size_t)b * p.maxblk + blk] * p.bs + (idx - (idx / p.bs) * p.bs);
+            row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
+            rows_lds[i] = (int)row;
+        }
     }
 
     f32x16 o[DVB];
@@ -167,56 +198,93 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     float m_run = -INFINITY;   // reference max, log2 domain
     float l_run = 0.f;         // running sum of exp2(s - m_run)
 
-    __syncthreads();
+    // gather registers of one tile: NP passes of two keys per wave (512 B int8 each), RP rope pieces
+    constexpr int NP = KT / (2 * NW);
+    constexpr int RP = (KT * (DR / 8)) / (NW * 64);
+    i32x4 raw[NP];
+    float rsc[NP];
+    u32x4 rrope[RP];
 
-    for (int kt = k_begin; kt < k_end; kt += KT) {
-        // ---- gather + de-quantise KT rows into LDS (each wave KT/NW rows, two rows per pass)
+    // wave w gathers keys w*KT/NW .. +KT/NW of the tile; within a pass the lower half-wave takes key
+    // half*NP + i, so a lane's NP row numbers are one contiguous LDS read
+    auto issue_loads = [&](const int kt) {
+        const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW) + half * NP;
 #pragma unroll
-        for (int i = 0; i < KT / (2 * NW); ++i) {
-            const int kl = w * (KT / NW) + 2 * i + half;
-            const bool valid = kt + kl < k_end;
-            const int row = valid ? rows_lds[kt - k_begin + kl] : 0;
-            i32x4 raw = {0, 0, 0, 0};
-            float sc = 0.f;
-            if (valid) {
-                raw = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * DN + 16 * col);
-                sc = p.ksc[(size_t)row * 4 + (col >> 3)];
-            }
-            dequant16(raw, sc, tile + kl * PITCH + 16 * col);
+        for (int i = 0; i < NP; ++i) {
+            const int row = rtab[i];
+            raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * DN + 16 * col);
+            rsc[i] = p.ksc[(size_t)row * 4 + (col >> 3)];
         }
-        for (int i = tid; i < KT * (DR / 8); i += NW * 64) {
-            const int kl = i >> 3;
-            const int part = i & 7;
-            const bool valid = kt + kl < k_end;
-            u32x4 v = {0, 0, 0, 0};
-            if (valid) {
-                const int row = rows_lds[kt - k_begin + kl];
-                v = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * DR + 8 * part);
-            }
-            *reinterpret_cast<u32x4 *>(tile + kl * PITCH + DN + 8 * part) = v;
+#pragma unroll
+        for (int i = 0; i < RP; ++i) {
+            const int e = tid + i * NW * 64;
+            const int row = rows_lds[(kt - k_begin) + (e >> 3)];
+            rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * DR + 8 * (e & 7));
         }
-        __syncthreads();
+    };
+    auto store_tile = [&](uint16_t *buf) {
+#pragma unroll
+        for (int i = 0; i < NP; ++i) {
+            const int kl = w * (KT / NW) + half * NP + i;
+            dequant16(raw[i], rsc[i], buf + kl * PITCH + 16 * col);
+        }
+#pragma unroll
+        for (int i = 0; i < RP; ++i) {
+            const int e = tid + i * NW * 64;
+            *reinterpret_cast<u32x4 *>(buf + (e >> 3) * PITCH + DN + 8 * (e & 7)) = rrope[i];
+        }
+    };
 
-        // ---- S^T = K . Q^T
+    __syncthreads();                       // row table complete
+    if (k_begin < k_end) {
+        issue_loads(k_begin);
+        store_tile(tile0);
+    }
+    __syncthreads();
+    // All global loads issued so far (Q^T fragments, first tile) are complete from here on, so that
+    // inside the loop the only outstanding vector-memory operations are the next tile's gather and
+    // the compiler's wait counts do not serialise it with the matrix products.
+    __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0), expcnt and lgkmcnt unconstrained
+
+    int it = 0;
+    for (int kt = k_begin; kt < k_end; kt += KT, ++it) {
+        const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
+        const bool has_next = kt + KT < k_end;
+        if (has_next) issue_loads(kt + KT);      // in flight during the matrix products below
+
+        // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
         {
-            const uint16_t *arow = tile + col * PITCH + 8 * half;
+            const uint16_t *arow = cur_tile + col * PITCH + 8 * half;
+            bf16x8 fa[2][4];
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                const bf16x8 a = *reinterpret_cast<const bf16x8 *>(arow + 16 * ks);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s, 0, 0, 0);
-                if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            for (int e = 0; e < 4; ++e) fa[0][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * e);
+#pragma unroll
+            for (int g = 0; g < KSTEPS / 4; ++g) {
+                if (g + 1 < KSTEPS / 4) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        fa[(g + 1) & 1][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * (4 * (g + 1) + e));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[g & 1][e], qf[4 * g + e], s, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
 
         // ---- online softmax; lane (head, half) holds keys kt + 8*(r/4) + 4*half + r%4
         float mx = -INFINITY;
+        if (kt + KT > k_end) {                  // only the split's last tile can hold keys past k_end
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (kt + 8 * (r >> 2) + 4 * half + (r & 3) >= k_end) s[r] = -INFINITY;
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int key = kt + 8 * (r >> 2) + 4 * half + (r & 3);
-            s[r] = key < k_end ? s[r] * p.scale_log2 : -INFINITY;
+            s[r] *= p.scale_log2;
             mx = fmaxf(mx, s[r]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -224,12 +292,12 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         // fp32 sums and bf16 P hold without loss, and the accumulators are rescaled only on a jump.
         const bool upd = mx > m_run + RESCALE_TAU;          // always true on the first tile (m_run = -inf)
         const float m_new = upd ? mx : m_run;
-        const float alpha = upd ? exp2f(m_run - m_new) : 1.0f;
+        const float alpha = upd ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
         const bool rescale = upd && l_run > 0.f;            // nothing accumulated yet: nothing to rescale
         float lsum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            s[r] = exp2f(s[r] - m_new);
+            s[r] = __builtin_amdgcn_exp2f(s[r] - m_new);      // v_exp_f32; exp2(-inf) = 0
             lsum += s[r];
         }
         lsum += __shfl_xor(lsum, 32);
@@ -249,81 +317,148 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             pf[kk] = __builtin_bit_cast(bf16x8, pk);
         }
 
-        // ---- O^T += V^T . P^T
+        // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead
         {
-            const uint16_t *vbase = tile + (4 * half + ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
-            AccLoop<0, DVB>::pv(o, vbase, pf[0]);
-            AccLoop<0, DVB>::pv(o, vbase + 16 * PITCH, pf[1]);
+            const uint16_t *vbase = cur_tile + (4 * half + ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+            s16x4 va[2][4][2];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                va[0][e][0] = lds_read_tr16(vbase + 32 * e);
+                va[0][e][1] = lds_read_tr16(vbase + 32 * e + 8 * PITCH);
+            }
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                if (g + 1 < 8) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int m = 4 * (g + 1) + e;
+                        const uint16_t *a0 = vbase + (16 * (m >> 4)) * PITCH + 32 * (m & 15);
+                        va[(g + 1) & 1][e][0] = lds_read_tr16(a0);
+                        va[(g + 1) & 1][e][1] = lds_read_tr16(a0 + 8 * PITCH);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = 4 * g + e;
+                    const s16x8 a = __builtin_shufflevector(va[g & 1][e][0], va[g & 1][e][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf[m >> 4]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
+
+        if (has_next) store_tile((it & 1) ? tile0 : tile1);
         __syncthreads();
     }
 
-    // ---- epilogue: lane (head, half) holds value channels 32*dvb + 8*(r/4) + 4*half + r%4
-    if (!head_ok) return;
+    // ---- epilogue.  Lane (head, half) holds value channels 32*dvb + 8*(r/4) + 4*half + r%4 of its head;
+    // written from there each store instruction would touch 32 rows with 32 bytes each.  Each wave
+    // instead transposes 128 channels at a time through its own slice of the (now idle) tile
+    // memory, so that 32 lanes write 512 contiguous bytes of one head (256 for the bf16 result).
     mfma_to_valu_fence();
-    if (p.nsplit == 1) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-        uint16_t *orow = p.out + ((size_t)t * p.NQ + head) * DN + 4 * half;
+    {
+        // staging slice of this wave: 32 heads x 128 channels fp32, 16-byte chunk c of head h stored at
+        // chunk c ^ (h & 7): both the column-wise writes and the row-wise reads are bank-conflict free.
+        // The accumulators go to LDS as they are (the 1/l factor is applied on the way out, from a
+        // small per-head table), and the way out is a rolled loop: the straight-line part of the
+        // epilogue is one LDS store per four accumulator registers.
+        float *stage = reinterpret_cast<float *>(pool) + w * (32 * 128);
+        float *inv_tab = reinterpret_cast<float *>(rows_lds) + w * 32;      // the row table is dead by now
+        const int head_base = hg * (32 * NW) + w * 32;
+        const size_t prow_base = ((size_t)t * p.nsplit + sp) * p.NQ;
+        if (half == 0) inv_tab[col] = l_run > 0.f ? 1.0f / l_run : 0.f;
+        // FINAL: bf16 result rows; otherwise fp16 partial of a key split (O / l of the split, merged by
+        // the combine kernel with weights l * 2^(m - m_max); O / l is a convex combination of
+        // de-quantised V rows, so it stays finite in fp16 as long as |int8 * scale| < 65504).
+        // ALL: every head of this wave exists, so the stores need no predicate.  Both are uniform
+        // and resolved outside the loops: scalar branches inside them cost more than the work.
+        auto drain = [&](auto final_tag, auto all_tag) {
+            constexpr bool FINAL = decltype(final_tag)::value;
+            constexpr bool ALL = decltype(all_tag)::value;
+            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 4 * col
+                                   : p.part_o + (prow_base + head_base + half) * DN + 4 * col;
 #pragma unroll
-        for (int dvb = 0; dvb < DVB; ++dvb)
+            for (int gq = 0; gq < DVB / 4; ++gq) {
 #pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                u32x2 v;
-                v[0] = pack_bf16x2(o[dvb][4 * q4] * inv, o[dvb][4 * q4 + 1] * inv);
-                v[1] = pack_bf16x2(o[dvb][4 * q4 + 2] * inv, o[dvb][4 * q4 + 3] * inv);
-                *reinterpret_cast<u32x2 *>(orow + 32 * dvb + 8 * q4) = v;
+                for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const f32x16 &acc = o[4 * gq + b4];
+                        const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
+                        *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
+                    }
+#pragma unroll 1
+                for (int pq = 0; pq < 2; ++pq) {
+                    f32x4 rv[8];
+                    float iv[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int hl = 2 * (8 * pq + e) + half;
+                        rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
+                        iv[e] = inv_tab[hl];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int hl = 2 * (8 * pq + e) + half;
+                        const f32x4 v = rv[e] * iv[e];
+                        u32x2 pk;
+                        pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
+                        pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
+                        if (ALL || head_base + hl < p.NQ)
+                            *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN + 128 * gq) = pk;
+                    }
+                }
             }
-    } else {
-        const size_t prow = ((size_t)t * p.nsplit + sp) * p.NQ + head;
-        float *po = p.part_o + prow * DN + 4 * half;
-#pragma unroll
-        for (int dvb = 0; dvb < DVB; ++dvb)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) {
-                f32x4 v = {o[dvb][4 * q4], o[dvb][4 * q4 + 1], o[dvb][4 * q4 + 2], o[dvb][4 * q4 + 3]};
-                *reinterpret_cast<f32x4 *>(po + 32 * dvb + 8 * q4) = v;
-            }
-        if (half == 0) {
-            p.part_ml[prow * 2] = m_run;
-            p.part_ml[prow * 2 + 1] = l_run;
+        };
+        const bool all_heads = head_base + 32 <= p.NQ;
+        if (p.nsplit == 1) {
+            if (all_heads) drain(std::true_type{}, std::true_type{});
+            else drain(std::true_type{}, std::false_type{});
+        } else {
+            if (all_heads) drain(std::false_type{}, std::true_type{});
+            else drain(std::false_type{}, std::false_type{});
+        }
+        if (p.nsplit > 1 && half == 0 && head_ok) {
+            p.part_ml[(prow_base + head) * 2] = m_run;
+            p.part_ml[(prow_base + head) * 2 + 1] = l_run;
         }
     }
 }
 
-// Merges the key splits of one query row: out = sum_s 2^(m_s - m) acc_s / sum_s 2^(m_s - m) l_s.
-// One thread per (row, head, 4 value channels).
+// Merges the key splits of one query row: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - m)
+// and O_s the split's normalised fp16 partial.  One thread per (row, head, 8 value channels).
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
 {
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t total = (size_t)p.T * p.NQ * (DN / 4);
+    const size_t total = (size_t)p.T * p.NQ * (DN / 8);
     if (gid >= total) return;
-    const int c4 = (int)(gid % (DN / 4));
-    const size_t th = gid / (DN / 4);
+    const int c8 = (int)(gid % (DN / 8));
+    const size_t th = gid / (DN / 8);
     const int head = (int)(th % p.NQ);
     const int t = (int)(th / p.NQ);
     float m = -INFINITY;
     for (int s = 0; s < p.nsplit; ++s) {
         const size_t prow = ((size_t)t * p.nsplit + s) * p.NQ + head;
-        m = fmaxf(m, p.part_ml[prow * 2]);
+        if (p.part_ml[prow * 2 + 1] > 0.f) m = fmaxf(m, p.part_ml[prow * 2]);
     }
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    float lsum = 0.f;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float wsum = 0.f;
     for (int s = 0; s < p.nsplit; ++s) {
         const size_t prow = ((size_t)t * p.nsplit + s) * p.NQ + head;
-        const float ms = p.part_ml[prow * 2];
         const float ls = p.part_ml[prow * 2 + 1];
         if (ls > 0.f) {
-            const float wgt = exp2f(ms - m);
-            const f32x4 v = *reinterpret_cast<const f32x4 *>(p.part_o + prow * DN + 4 * c4);
-            acc += v * wgt;
-            lsum += ls * wgt;
+            const float wgt = ls * __builtin_amdgcn_exp2f(p.part_ml[prow * 2] - m);
+            const f16x8 hv = *reinterpret_cast<const f16x8 *>(p.part_o + prow * DN + 8 * c8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += wgt * (float)hv[e];
+            wsum += wgt;
         }
     }
-    const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-    u32x2 v;
-    v[0] = pack_bf16x2(acc[0] * inv, acc[1] * inv);
-    v[1] = pack_bf16x2(acc[2] * inv, acc[3] * inv);
-    *reinterpret_cast<u32x2 *>(p.out + ((size_t)t * p.NQ + head) * DN + 4 * c4) = v;
+    const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+    u32x4 v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = pack_bf16x2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+    *reinterpret_cast<u32x4 *>(p.out + ((size_t)t * p.NQ + head) * DN + 8 * c8) = v;
 }
 
 }  // namespace
@@ -340,7 +475,7 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.nsplit > 1) {
-        const size_t total = (size_t)p.T * p.NQ * (DN / 4);
+        const size_t total = (size_t)p.T * p.NQ * (DN / 8);
         hipLaunchKernelGGL(sfa_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
         e = hipGetLastError();
     }
