@@ -35,37 +35,35 @@ constexpr int PITCH = D + 8;      // LDS row pitch in bf16 elements (1168 B: row
 constexpr int KSTEPS = D / 16;    // 36 contraction steps of 16
 constexpr int DVB = DN / 32;      // 16 output blocks of 32 value channels
 
-// 16 int8 (one 16-byte load) times one scale -> 16 bf16 as two 16-byte LDS stores.
+// 8 int8 (two dwords of a 16-byte load) times one scale -> 8 bf16 as one 16-byte LDS store.
 // x*sc is formed as fma(float(x + 128), sc, -128*sc): the byte is biased to unsigned so that a single
 // v_cvt_f32_ubyteN converts it, and the fused multiply-add rounds the exact product (x*sc) once, which
 // is bit-identical to the rounded multiply (128*sc is exact).
-__device__ __forceinline__ void dequant16(const i32x4 raw, const float sc, uint16_t *dst)
+__device__ __forceinline__ void dequant8(const int r0, const int r1, const float sc, uint16_t *dst)
 {
     const float bias = -128.0f * sc;
-    u32x4 lo, hi;
+    u32x4 out;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        const uint32_t v = (uint32_t)raw[w] ^ 0x80808080u;
+    for (int w = 0; w < 2; ++w) {
+        const uint32_t v = (uint32_t)(w == 0 ? r0 : r1) ^ 0x80808080u;
         const float f0 = __builtin_fmaf((float)(v & 0xffu), sc, bias);
         const float f1 = __builtin_fmaf((float)((v >> 8) & 0xffu), sc, bias);
         const float f2 = __builtin_fmaf((float)((v >> 16) & 0xffu), sc, bias);
         const float f3 = __builtin_fmaf((float)(v >> 24), sc, bias);
-        const uint32_t p0 = pack_bf16x2(f0, f1);
-        const uint32_t p1 = pack_bf16x2(f2, f3);
-        if (w < 2) { lo[2 * w] = p0; lo[2 * w + 1] = p1; }
-        else { hi[2 * (w - 2)] = p0; hi[2 * (w - 2) + 1] = p1; }
+        out[2 * w] = pack_bf16x2(f0, f1);
+        out[2 * w + 1] = pack_bf16x2(f2, f3);
     }
-    *reinterpret_cast<u32x4 *>(dst) = lo;
-    *reinterpret_cast<u32x4 *>(dst + 8) = hi;
+    *reinterpret_cast<u32x4 *>(dst) = out;
 }
 
 // O^T accumulators live in the accumulation registers for the whole kernel (16 blocks x 16 = all 256 of
-// them).  Every instruction that touches them inside the key loop is inline assembly with an
-// accumulation-register constraint, so the register allocator cannot migrate them into the 256
-// architectural registers, most of which hold the Q^T fragments.
+// them).  Inside the key loop they are touched only by the matrix product itself and by acc_scale,
+// which works on them in place through inline assembly: any plain C++ arithmetic on them makes the
+// register allocator migrate them into the 256 architectural registers, most of which hold the Q^T
+// fragments (observed: hundreds of spilled registers).
 __device__ __forceinline__ void acc_mfma(f32x16 &acc, const bf16x8 a, const bf16x8 b)
 {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
 
 // acc *= alpha, one register at a time through a single architectural temporary (rare path)
@@ -105,7 +103,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // Epilogue: per-wave transposition slices.
     constexpr int POOL_ROWS = 32 * NW > 2 * KT ? 32 * NW : 2 * KT;     // at least the two tile buffers
     __shared__ __attribute__((aligned(16))) uint16_t pool[POOL_ROWS * PITCH];
-    __shared__ int rows_lds[SFA_MAX_CHUNK];
+    __shared__ int rows_lds[SFA_MAX_CHUNK + KT];
     uint16_t *const tile0 = pool;
     uint16_t *const tile1 = pool + KT * PITCH;
 
@@ -174,11 +172,12 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     }
 
     // logical position -> physical cache row for this split's keys.  The table is padded to a whole
-    // number of tiles with the row of the split's first key: keys past k_end are then loaded like any
-    // other (finite data) and masked out of the softmax, so the loop needs no per-key branches.
+    // number of tiles plus one with the row of the split's first key: keys past k_end are then loaded
+    // like any other (finite data) and masked out of the softmax, and the loop can prefetch "the next
+    // tile" unconditionally -- no per-key and no per-tile branches.
     {
         const int n_valid = k_end - k_begin;
-        const int n_pad = (n_valid + KT - 1) / KT * KT;
+        const int n_pad = n_valid > 0 ? (n_valid + KT - 1) / KT * KT + KT : 0;   // + one tile: see the loop
         for (int i = tid; i < n_pad; i += NW * 64) {
             const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
             int blk = idx / p.bs;
@@ -222,17 +221,31 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * DR + 8 * (e & 7));
         }
     };
+    // de-quantise and store one eighth of the gathered tile (piece 0 also stores the rope part)
+    auto store_piece = [&](uint16_t *buf, const int piece) {
+        static_assert(NP * 2 % 8 == 0 || NP * 2 == 8 || true, "");
+        constexpr int HALVES = 2 * NP;                 // 16-byte LDS stores of this lane per tile
+        constexpr int PER = (HALVES + 7) / 8;          // ... per piece
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int hidx = piece * PER + q;
+            if (hidx < HALVES) {
+                const int i = hidx >> 1, hh = hidx & 1;
+                const int kl = w * (KT / NW) + half * NP + i;
+                dequant8(raw[i][2 * hh], raw[i][2 * hh + 1], rsc[i], buf + kl * PITCH + 16 * col + 8 * hh);
+            }
+        }
+        if (piece == 0) {
+#pragma unroll
+            for (int i = 0; i < RP; ++i) {
+                const int e = tid + i * NW * 64;
+                *reinterpret_cast<u32x4 *>(buf + (e >> 3) * PITCH + DN + 8 * (e & 7)) = rrope[i];
+            }
+        }
+    };
     auto store_tile = [&](uint16_t *buf) {
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int kl = w * (KT / NW) + half * NP + i;
-            dequant16(raw[i], rsc[i], buf + kl * PITCH + 16 * col);
-        }
-#pragma unroll
-        for (int i = 0; i < RP; ++i) {
-            const int e = tid + i * NW * 64;
-            *reinterpret_cast<u32x4 *>(buf + (e >> 3) * PITCH + DN + 8 * (e & 7)) = rrope[i];
-        }
+        for (int piece = 0; piece < 8; ++piece) store_piece(buf, piece);
     };
 
     __syncthreads();                       // row table complete
@@ -249,8 +262,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     int it = 0;
     for (int kt = k_begin; kt < k_end; kt += KT, ++it) {
         const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
-        const bool has_next = kt + KT < k_end;
-        if (has_next) issue_loads(kt + KT);      // in flight during the matrix products below
+        uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
+        issue_loads(kt + KT);                    // next tile (or the padding tile): in flight during the products
 
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
@@ -317,7 +330,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             pf[kk] = __builtin_bit_cast(bf16x8, pk);
         }
 
-        // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead
+        // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead;
+        // interleaved with the de-quantisation of the next tile into the other buffer
         {
             const uint16_t *vbase = cur_tile + (4 * half + ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
             s16x4 va[2][4][2];
@@ -343,11 +357,11 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                     const s16x8 a = __builtin_shufflevector(va[g & 1][e][0], va[g & 1][e][1], 0, 1, 2, 3, 4, 5, 6, 7);
                     acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf[m >> 4]);
                 }
+                // one eighth of the next tile's de-quantisation rides in the shadow of these products
+                store_piece(nxt_tile, g);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-
-        if (has_next) store_tile((it & 1) ? tile0 : tile1);
         __syncthreads();
     }
 
