@@ -115,9 +115,9 @@ int li_check(const PtoLiDecodeArgs *a)
 
 size_t li_ws_bytes(const PtoLiDecodeArgs *a)
 {
-    // score rows [t, max_blocknum_perbatch*block_size] fp32 + w_scale [t, 64] fp32
+    // score rows [t, max_blocknum_perbatch*block_size] fp32
     const size_t stride = (size_t)a->max_blocknum_perbatch * a->block_size;
-    return (size_t)a->t * stride * sizeof(float) + (size_t)a->t * 64 * sizeof(float);
+    return (size_t)a->t * stride * sizeof(float);
 }
 
 }  // namespace
@@ -216,11 +216,14 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.k = (int)a->selected_count;
     p.score_stride = (long long)a->max_blocknum_perbatch * a->block_size;
     p.scores = static_cast<float *>(a->workspace);
-    p.w_scale = p.scores + (size_t)a->t * p.score_stride;
     p.q_dt = a->q_scale_dtype;
     p.k_dt = a->k_scale_dtype;
     p.w_dt = a->weight_dtype;
-    p.num_cu = cu_count();
+    {   // enough waves to cover every SIMD a few times, at most 8 blocks (256 keys) per wave
+        const long long blocks = (long long)a->t * ((p.score_stride + 31) / 32);
+        long long bpw = blocks / ((long long)cu_count() * 4 * 4);
+        p.bpw = (int)(bpw < 1 ? 1 : (bpw > 8 ? 8 : bpw));
+    }
     hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;

@@ -20,11 +20,10 @@ struct LiParams {
     const int32_t *bt;      // [B, maxblk]
     int32_t *topk_res;      // [T, k]
     float *scores;          // workspace [T, score_stride]
-    float *w_scale;         // workspace [T, 64]
     long long score_stride;
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes
-    int num_cu;
+    int bpw;                // 32-key blocks per wave of the score kernel
 };
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream);
