@@ -15,11 +15,14 @@
 //                     token's 64 query heads (two 32-row operands resident in registers) and
 //                     B = 32 key rows loaded straight from the paged cache in operand layout;
 //                     epilogue in registers; scores to a [T, max_seq] fp32 workspace
-//   li_select_kernel  one workgroup per query token, score keys resident in registers: 3-pass radix
-//                     select (11+11+10 bits) on an order-preserving 32-bit image of the score, a
-//                     position select among candidates tied at the threshold, bitonic sort of the
-//                     survivors by (score desc, position asc); li_select_stream_kernel is the
-//                     memory-streaming form for rows longer than 65536
+//   li_select_kernel  one workgroup per query token, keys ordered by the strict word
+//                     (score image << 32 | ~position): a histogram of a 2048-score sample gives a
+//                     pivot, one pass over the row compacts the keys above it, those are spread over
+//                     2048 buckets linear in the score and ordered inside buckets by counting;
+//                     select_streaming (radix select over the row in memory + bitonic sort) is the
+//                     capacity-free form it falls back to
+#include <type_traits>
+
 #include "common.h"
 #include "li_kernels.h"
 #include "pypto_amd_sfa.h"
@@ -67,9 +70,6 @@ __device__ __forceinline__ uint32_t score_key(const float x)
     u = u == 0x80000000u ? 0u : u;
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
-
-constexpr int HIST_BITS = 13;                 // first-level histogram: the top 13 bits of the key
-constexpr int HIST_BINS = 1 << HIST_BITS;
 
 __global__ __launch_bounds__(256) void li_score_kernel(const LiParams p)
 {
@@ -379,21 +379,11 @@ __device__ void bitonic_sort_desc(unsigned long long *buf, const int width, cons
     __syncthreads();
 }
 
-constexpr int SEL_CAP = 4096;       // keys of the threshold bin the fast path holds in LDS
-constexpr int SEL_RANK_MAX = 512;   // longest bin segment ordered by counting; longer ones use the bitonic sort
-constexpr int SEL_DIRECT_MAX = 256; // most threshold-bin keys resolved by counting instead of radix passes
+constexpr int SEL_SAMPLE = 2048;   // most keys sampled from a row
+constexpr int SEL_CAP = 8192;      // candidates (keys above the pivot) the fast path holds in LDS
+constexpr int SEL_STAGE = 4096;    // entries of the buckets down to the one holding the k-th best
+constexpr int SEL_RANK_MAX = 512;  // rows of at most k keys: ordered by counting up to this length, else sorted
 
-// One workgroup per query token.
-//   pass 1 over the row: histogram of the top 13 key bits (LDS) -> the bin holding the k-th best key,
-//           how many keys to take inside it, and the output offset of every bin above it;
-//   pass 2 over the row: keys above that bin are scattered straight into their bin's output range,
-//           keys inside it go to a candidate list;
-//   candidates: few -> ordered by counting; many -> two 10-bit radix passes for the exact key of the
-//           k-th best plus, if more candidates tie at that key than are needed, two passes over
-//           their positions (lowest positions win);
-//   each bin's range is then ordered by counting (every key counts the larger keys of its range).
-// Order is (key desc, position asc) throughout: the 64-bit word (key << 32) | ~position, descending.
-// A threshold bin with more than SEL_CAP keys takes the general streaming path.
 // how many entries of list[beg, end) are larger than e; eight LDS reads in flight per round
 __device__ __forceinline__ uint32_t count_greater(const unsigned long long *list, const uint32_t beg, const uint32_t end,
                                                   const unsigned long long e)
@@ -409,16 +399,103 @@ __device__ __forceinline__ uint32_t count_greater(const unsigned long long *list
     return rank;
 }
 
+// the 64-bit word whose descending order is (score descending, position ascending); never zero
+__device__ __forceinline__ unsigned long long order_word(const float score, const uint32_t pos)
+{
+    return ((unsigned long long)score_key(score) << 32) | (uint32_t)(~pos);
+}
+
+// Wave-wide scan and reductions on DPP (no LDS traffic).  row_shr:n moves a value n lanes up inside
+// its row of 16, row_bcast15/31 carry the last lane of a row / of the lower half-wave upward; lanes
+// without a source keep the identity passed as the old value.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_u32(const uint32_t identity, const uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)identity, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// inclusive prefix sum over the 64 lanes
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v)
+{
+    v += dpp_u32<0x111, 0xf>(0u, v);
+    v += dpp_u32<0x112, 0xf>(0u, v);
+    v += dpp_u32<0x114, 0xf>(0u, v);
+    v += dpp_u32<0x118, 0xf>(0u, v);
+    v += dpp_u32<0x142, 0xa>(0u, v);
+    v += dpp_u32<0x143, 0xc>(0u, v);
+    return v;
+}
+
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_reduce_bits(uint32_t v, const uint32_t identity, Op op)
+{
+    v = op(v, dpp_u32<0x111, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x112, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x114, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x118, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x142, 0xa>(identity, v));
+    v = op(v, dpp_u32<0x143, 0xc>(identity, v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);     // lane 63 holds the reduction of all lanes
+}
+
+__device__ __forceinline__ float wave_min(const float x)
+{
+    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0x7f800000u, [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fminf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
+__device__ __forceinline__ float wave_max(const float x)
+{
+    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0xff800000u, [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(const uint32_t x)
+{
+    return wave_reduce_bits(x, 0u, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+}
+
+// score whose order-preserving image is key (the inverse of score_key)
+__device__ __forceinline__ float key_score(const uint32_t key)
+{
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+constexpr int SEL_SBINS = 1024;    // bins of the sample histogram
+constexpr int SEL_BUCKETS = 2048;  // buckets the candidates are spread over
+constexpr int SEL_WAVE_CAP = SEL_CAP / SEL_WAVES;   // candidates one wave can compact
+constexpr int SEL_CHUNK = 32 * SEL_THREADS;   // scores one trip of the row scan holds in registers
+
+// One workgroup per query token: a distribution-adaptive bucket select.  Every key is ordered by the
+// word (score image << 32) | ~position, a strict order, so ties need no special case.
+//   1. up to 2048 scores are sampled (one per stratum of the row, jittered).  A histogram of the
+//      sample over [sample min, sample max] gives the pivot: the lower edge of the bin in which the
+//      sample reaches rank r = r0 + 6*sqrt(r0) + 8, r0 = k*S/n.  With overwhelming probability at
+//      least k and at most SEL_CAP scores of the row lie at or above it;
+//   2. one pass over the row (32 scores per thread in flight at once, requested before the sample is
+//      looked at) compacts the keys at or above the pivot into a candidate list;
+//   3. the candidates are spread over 2048 buckets linear in the score between the pivot and the
+//      sample maximum, bucket 0 highest: bins follow the values instead of the float encoding, so
+//      the counters see few collisions and buckets stay short whatever the scale of the scores;
+//   4. a prefix sum over the bucket counts finds the bucket holding the k-th best key; the buckets
+//      down to it are staged contiguously and each is ordered by counting (a key's rank = the number
+//      of larger keys of its bucket).  Output slots below k are written straight to memory.
+// If the pivot misjudges the row (fewer than k candidates, more than the list holds, or a bucket
+// range too long to stage) the general streaming select runs instead.
 __global__ __launch_bounds__(SEL_THREADS) void li_select_kernel(const LiParams p)
 {
-    __shared__ uint32_t hist[HIST_BINS];      // keys per first-level bin
-    __shared__ uint32_t rhist[1024];          // histogram of the radix passes over the candidates
-    __shared__ uint32_t cursor[HIST_BINS];    // next free output slot of each bin above the threshold bin
-    __shared__ unsigned long long stage[LI_MAX_SELECT];   // survivors grouped by bin, unordered inside
-    __shared__ unsigned long long sortbuf[LI_MAX_SELECT];
-    __shared__ unsigned long long cand[SEL_CAP];
+    __shared__ unsigned long long cand[SEL_CAP + 64];  // + one dump slot per lane
+    __shared__ unsigned long long stage[SEL_STAGE];    // also the sort buffer of the other paths
+    __shared__ uint16_t sbucket[SEL_STAGE];            // bucket of every staged entry
+    __shared__ uint32_t bcount[SEL_BUCKETS];
+    __shared__ uint32_t boff[SEL_BUCKETS];
+    __shared__ uint32_t shist[SEL_SBINS];
+    __shared__ uint32_t hist[256];                     // streaming path only
     __shared__ uint32_t wave_tot[SEL_WAVES];
-    __shared__ uint32_t sh_prefix, sh_krem, sh_ncand, sh_nsurv, sh_longest;
+    __shared__ float wave_mn[SEL_WAVES], wave_mx[SEL_WAVES];
+    __shared__ uint32_t sh_over, sh_tb;
 
     const int t = blockIdx.x;
     const int b = t / p.S1;
@@ -434,264 +511,262 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_kernel(const LiParams p
     const int k = p.k;
     const float *srow = p.scores + (size_t)t * p.score_stride;
     int32_t *out = p.topk_res + (size_t)t * k;
-    const int nsel = n < k ? n : k;
 
-    // histogram of `digit` over the lanes with `act`; a digit shared by all of them costs one add
-    auto hist_add = [&](uint32_t *h, const bool act, const uint32_t digit) {
-        const unsigned long long m = __ballot(act);
-        if (m == 0ull) return;
-        const int first = __ffsll((long long)m) - 1;
-        const uint32_t d = __shfl(digit, first);
-        if (__ballot(act && digit == d) == m) {
-            if (lane == first) atomicAdd(&h[d], (uint32_t)__popcll(m));
-        } else if (act) {
-            atomicAdd(&h[digit], 1u);
-        }
-    };
-    // Bins of hist[] visited from the top (descending) or the bottom, eight per thread; finds the bin
-    // holding the krem-th element and how many remain to be taken inside it.  nbins <= 8192.
-    // With offsets != nullptr also records, for every bin, how many elements precede it.
-    auto pick_bin = [&](const uint32_t *h, const int nbins, const bool descending, const uint32_t krem, uint32_t &bin,
-                        uint32_t &rest, uint32_t *offsets) {
-        uint32_t c[8];
-        int idx[8];
-        uint32_t tot = 0;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int v = 8 * tid + e;                        // visiting order
-            idx[e] = descending ? nbins - 1 - v : v;
-            c[e] = v < nbins ? h[idx[e]] : 0u;
-            tot += c[e];
-        }
-        uint32_t incl = tot;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const uint32_t v = __shfl_up(incl, off);
-            if (lane >= off) incl += v;
-        }
-        if (lane == 63) wave_tot[wv] = incl;
-        __syncthreads();
-        uint32_t before = incl - tot;
-        for (int i = 0; i < wv; ++i) before += wave_tot[i];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (offsets != nullptr && 8 * tid + e < nbins) offsets[idx[e]] = before;
-            if (before < krem && krem <= before + c[e]) { sh_prefix = (uint32_t)idx[e]; sh_krem = krem - before; }
-            before += c[e];
-        }
-        __syncthreads();
-        bin = sh_prefix;
-        rest = sh_krem;
-        __syncthreads();
-    };
-
-    if (tid == 0) { sh_ncand = 0; sh_nsurv = 0; sh_longest = 0; }
     if (n <= k) {
-        // everything is selected: one range, ordered below
-        for (int i = tid; i < n; i += SEL_THREADS)
-            stage[i] = ((unsigned long long)score_key(srow[i]) << 32) | (uint32_t)(~(uint32_t)i);
-        __syncthreads();
+        // everything is selected; the tail of the output row is padding
+        for (int i = n + tid; i < k; i += SEL_THREADS) out[i] = -1;
         if (n > SEL_RANK_MAX) {
             int width = 64;
             while (width < n) width <<= 1;
-            for (int i = tid; i < width; i += SEL_THREADS) sortbuf[i] = i < n ? stage[i] : 0ull;
+            for (int i = tid; i < width; i += SEL_THREADS) stage[i] = i < n ? order_word(srow[i], (uint32_t)i) : 0ull;
             __syncthreads();
-            bitonic_sort_desc(sortbuf, width, tid);
+            bitonic_sort_desc(stage, width, tid);
+            for (int i = tid; i < n; i += SEL_THREADS) out[i] = (int32_t)(~(uint32_t)stage[i]);
         } else {
+            for (int i = tid; i < n; i += SEL_THREADS) stage[i] = order_word(srow[i], (uint32_t)i);
+            __syncthreads();
             for (int i = tid; i < n; i += SEL_THREADS) {
                 const unsigned long long e = stage[i];
-                sortbuf[count_greater(stage, 0u, (uint32_t)n, e)] = e;
+                out[count_greater(stage, 0u, (uint32_t)n, e)] = (int32_t)(~(uint32_t)e);
             }
-            __syncthreads();
         }
-    } else {
-        // Both passes over the row are rolled loops (the kernel runs once per token, so straight-line
-        // code would be fetched cold) with the next round's eight loads in flight while a round is
-        // processed.
-        constexpr int U = 8;
-        auto load_round = [&](const int i0, float (&v)[U]) {
+        return;
+    }
+
+    // ---- 1. sample: the loads go out first, then the first chunk of the row, so that one memory
+    // latency covers both
+    const uint32_t S = n < SEL_SAMPLE ? (uint32_t)n : (uint32_t)SEL_SAMPLE;
+    float sx[2];
+    bool sval[2];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = i0 + u * SEL_THREADS + tid;
-                v[u] = srow[i < n ? i : n - 1];
+    for (int e = 0; e < 2; ++e) {
+        const uint32_t i = (uint32_t)(tid + e * SEL_THREADS);
+        sval[e] = i < S;
+        // stratum i of the row is [i*n/S, (i+1)*n/S): products stay below 2^28
+        const uint32_t ic = sval[e] ? i : 0u;
+        const uint32_t lo = ic * (uint32_t)n / S, hi = (ic + 1u) * (uint32_t)n / S;
+        sx[e] = srow[lo + ((ic * 2654435761u) >> 16) % (hi - lo)];
+    }
+    // the row as 16-byte vectors: thread tid holds vectors u*1024 + tid of a chunk.  The row buffer is
+    // score_stride (a multiple of 32) long, so whole vectors stay inside it.
+    const int last_vec = (int)(p.score_stride >> 2) - 1;
+    auto load_chunk = [&](const int c0, f32x4 (&v)[8]) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int vi = (c0 >> 2) + u * SEL_THREADS + tid;
+            v[u] = reinterpret_cast<const f32x4 *>(srow)[vi < last_vec ? vi : last_vec];
+        }
+    };
+    f32x4 v[8], vn[8];
+    load_chunk(0, v);
+
+    for (int i = tid; i < SEL_SBINS; i += SEL_THREADS) shist[i] = 0u;
+    for (int i = tid; i < SEL_BUCKETS; i += SEL_THREADS) bcount[i] = 0u;
+    if (tid == 0) sh_over = 0u;
+    {
+        float mn = __builtin_inff(), mx = -__builtin_inff();
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+            if (sval[e]) { mn = fminf(mn, sx[e]); mx = fmaxf(mx, sx[e]); }
+        mn = wave_min(mn);
+        mx = wave_max(mx);
+        if (lane == 0) { wave_mn[wv] = mn; wave_mx[wv] = mx; }
+    }
+    __syncthreads();
+    float smin = wave_mn[0], smax = wave_mx[0];
+#pragma unroll
+    for (int i = 1; i < SEL_WAVES; ++i) { smin = fminf(smin, wave_mn[i]); smax = fmaxf(smax, wave_mx[i]); }
+    const uint32_t r0 = ((uint32_t)k * S + (uint32_t)n - 1u) / (uint32_t)n;
+    const uint32_t r = r0 + (uint32_t)(6.0f * __builtin_sqrtf((float)r0)) + 8u;
+    float pivot = -__builtin_inff();       // candidates: score >= pivot
+    float blo = smin;                      // lower edge of the lowest bucket
+    if (r < S) {
+        const float range = smax - smin;
+        const float sscale = range > 0.f ? (float)SEL_SBINS / range : 0.f;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            if (sval[e]) {
+                const uint32_t sb = (uint32_t)fmaxf((sx[e] - smin) * sscale, 0.f);
+                atomicAdd(&shist[sb < (uint32_t)SEL_SBINS ? sb : (uint32_t)SEL_SBINS - 1u], 1u);
             }
-        };
-        // ---- pass 1: first-level histogram
-        for (int i = tid; i < HIST_BINS; i += SEL_THREADS) hist[i] = 0u;
+        }
         __syncthreads();
+        // every wave scans the 1024 bins from the top by itself (lane l owns the 16 bins below
+        // 1024 - 16*l): the bin in which the running count reaches r
+        uint32_t c[16];
+        uint32_t tot = 0;
         {
-            float v[U], vn[U];
-            load_round(0, v);
-            for (int i0 = 0; i0 < n; i0 += SEL_THREADS * U) {
-                load_round(i0 + SEL_THREADS * U, vn);
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(&shist[SEL_SBINS - 16 - 16 * lane]);
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    hist_add(hist, i0 + u * SEL_THREADS + tid < n, score_key(v[u]) >> (32 - HIST_BITS));
+            for (int q = 0; q < 4; ++q) {
+                const u32x4 x = src[q];
+                c[4 * q] = x[0]; c[4 * q + 1] = x[1]; c[4 * q + 2] = x[2]; c[4 * q + 3] = x[3];
+            }
 #pragma unroll
-                for (int u = 0; u < U; ++u) v[u] = vn[u];
+            for (int q = 0; q < 16; ++q) tot += c[q];
+        }
+        uint32_t before = wave_incl_scan(tot) - tot;
+        uint32_t pb = 0;                   // found by exactly one lane (the sample holds S >= r scores)
+#pragma unroll
+        for (int q = 15; q >= 0; --q) {
+            if (before < r && r <= before + c[q]) pb = (uint32_t)(SEL_SBINS - 16 - 16 * lane + q);
+            before += c[q];
+        }
+        pb = wave_max_u32(pb);
+        pivot = smin + (float)pb * (range * (1.0f / (float)SEL_SBINS));
+        blo = pivot;
+    }
+    // the buckets reach a quarter of the range past the sample maximum, so that the few scores above
+    // it spread out too; anything beyond shares bucket 0
+    const float bscale = smax - blo > 0.f ? (float)SEL_BUCKETS / (1.25f * (smax - blo)) : 0.f;
+
+    // ---- 2. candidates.  Wave w compacts the candidates among its keys into its own region of the
+    // list, cand[w*SEL_WAVE_CAP ...], so the waves share no counter.  A key costs a compare and an add
+    // to be counted and, branch-free, a compare, a select, an add and one LDS write of the raw
+    // (score bits, position) pair: a key that is no candidate goes to the lane's dump slot.  The
+    // order word is formed later, for the candidates only.  Wave-wide sums use DPP, not LDS.
+    uint32_t wave_count = 0;               // candidates of this wave so far (uniform)
+    auto scan_chunk = [&](const int c0, auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;          // the whole chunk lies inside the row
+        const int i_base = c0 + 4 * tid;
+        uint32_t mine = 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int i = i_base + 4 * u * SEL_THREADS + c;
+                mine += ((FULL || i < n) && v[u][c] >= pivot) ? 1u : 0u;
             }
         }
-        __syncthreads();
-        uint32_t bin0, rest;
-        pick_bin(hist, HIST_BINS, true, (uint32_t)k, bin0, rest, cursor);
-        const uint32_t n_bin = hist[bin0];
-        const uint32_t base0 = (uint32_t)k - rest;               // first output slot of the threshold bin
-        // longest range above the threshold bin (decides how the ranges are ordered)
-        {
-            uint32_t mx = 0;
-            for (int i = tid; i < HIST_BINS; i += SEL_THREADS)
-                if ((uint32_t)i > bin0) mx = hist[i] > mx ? hist[i] : mx;
-            if (mx > 0) atomicMax(&sh_longest, mx);
-        }
-        __syncthreads();
-        if (n_bin > (uint32_t)SEL_CAP) {
-            select_streaming(p, t, hist, sortbuf);               // uniform: the whole workgroup goes
+        const uint32_t incl = wave_incl_scan(mine);
+        const uint32_t wave_n = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+        if (wave_count + wave_n > (uint32_t)SEL_WAVE_CAP) {       // region overflow: the streaming path will run
+            if (lane == 0) sh_over = 1u;
             return;
         }
-        // ---- pass 2: scatter
-        {
-            float v[U], vn[U];
-            load_round(0, v);
-            for (int i0 = 0; i0 < n; i0 += SEL_THREADS * U) {
-                load_round(i0 + SEL_THREADS * U, vn);
-                uint32_t ncand_lane = 0;
-                unsigned long long cval[U];
+        uint32_t slot = (uint32_t)(wv * SEL_WAVE_CAP) + wave_count + incl - mine;
+        wave_count += wave_n;
+        const uint32_t dump = (uint32_t)(SEL_CAP + lane);
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int i = i0 + u * SEL_THREADS + tid;
-                    const uint32_t key = score_key(v[u]);
-                    const uint32_t kb = key >> (32 - HIST_BITS);
-                    const unsigned long long val = ((unsigned long long)key << 32) | (uint32_t)(~(uint32_t)i);
-                    if (i < n && kb > bin0) stage[atomicAdd(&cursor[kb], 1u)] = val;
-                    const bool is_c = i < n && kb == bin0;
-                    cval[u] = is_c ? val : 0ull;
-                    ncand_lane += is_c ? 1u : 0u;
-                }
-                // threshold-bin keys of the whole wave take one counter update
-                if (__ballot(ncand_lane != 0u) != 0ull) {
-                    uint32_t incl = ncand_lane;
+        for (int u = 0; u < 8; ++u) {
 #pragma unroll
-                    for (int off = 1; off < 64; off <<= 1) {
-                        const uint32_t x = __shfl_up(incl, off);
-                        if (lane >= off) incl += x;
-                    }
-                    const uint32_t wave_n = __shfl(incl, 63);
-                    uint32_t basec = 0;
-                    if (lane == 0) basec = atomicAdd(&sh_ncand, wave_n);
-                    basec = __shfl(basec, 0) + incl - ncand_lane;
-#pragma unroll
-                    for (int u = 0; u < U; ++u)
-                        if (cval[u] != 0ull) { if (basec < (uint32_t)SEL_CAP) cand[basec] = cval[u]; ++basec; }
-                }
-#pragma unroll
-                for (int u = 0; u < U; ++u) v[u] = vn[u];
+            for (int c = 0; c < 4; ++c) {
+                const int i = i_base + 4 * u * SEL_THREADS + c;
+                const bool is_c = (FULL || i < n) && v[u][c] >= pivot;
+                cand[is_c ? slot : dump] = ((unsigned long long)(uint32_t)i << 32) | __float_as_uint(v[u][c]);
+                slot += is_c ? 1u : 0u;
             }
         }
-        __syncthreads();
-        const uint32_t n_cand = sh_ncand < (uint32_t)SEL_CAP ? sh_ncand : (uint32_t)SEL_CAP;   // == n_bin
+    };
+    for (int c0 = 0; c0 < n; c0 += SEL_CHUNK) {
+        if (c0 + SEL_CHUNK < n) load_chunk(c0 + SEL_CHUNK, vn);
+        if (c0 + SEL_CHUNK <= n) scan_chunk(c0, std::true_type{});
+        else scan_chunk(c0, std::false_type{});
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = vn[u];
+    }
+    if (lane == 0) wave_tot[wv] = wave_count;
 
-        if (n_cand <= (uint32_t)SEL_DIRECT_MAX) {
-            // few candidates: a candidate's rank among them is its place in the bin's output range
-            for (uint32_t i = tid; i < n_cand; i += SEL_THREADS) {
-                const unsigned long long e = cand[i];
-                const uint32_t rank = count_greater(cand, 0u, n_cand, e);
-                if (rank < rest) sortbuf[base0 + rank] = e;
-            }
-        } else {
-            // ---- exact key of the k-th best among the candidates: the 32 - HIST_BITS low key bits in two
-            // radix passes (10 bits, then the rest)
-            uint32_t prefix = bin0 << (32 - HIST_BITS);
-            uint32_t krem = rest;
-            constexpr int LOW = 32 - HIST_BITS;
-#pragma unroll 1
-            for (int pass = 0; pass < 2; ++pass) {
-                const int shift = pass == 0 ? LOW - 10 : 0;
-                const int nbits = pass == 0 ? 10 : LOW - 10;
-                for (int i = tid; i < 1024; i += SEL_THREADS) rhist[i] = 0;
-                __syncthreads();
-                const uint32_t himask = 0xffffffffu << (shift + nbits);
-                for (uint32_t i0 = 0; i0 < n_cand; i0 += SEL_THREADS) {
-                    const uint32_t i = i0 + tid;
-                    const uint32_t key = i < n_cand ? (uint32_t)(cand[i] >> 32) : 0u;
-                    hist_add(rhist, i < n_cand && (key & himask) == prefix, (key >> shift) & ((1u << nbits) - 1u));
-                }
-                __syncthreads();
-                uint32_t bin;
-                pick_bin(rhist, 1 << nbits, true, krem, bin, krem, nullptr);
-                prefix |= bin << shift;
-            }
-            const uint32_t thr = prefix;
-            // ---- ties at thr: the krem lowest positions (17 position bits: 9 high, 8 low)
-            for (int i = tid; i < 512; i += SEL_THREADS) rhist[i] = 0;
-            __syncthreads();
-            for (uint32_t i0 = 0; i0 < n_cand; i0 += SEL_THREADS) {
-                const uint32_t i = i0 + tid;
-                const unsigned long long c = i < n_cand ? cand[i] : 0ull;
-                hist_add(rhist, i < n_cand && (uint32_t)(c >> 32) == thr, (~(uint32_t)c) >> 8);
-            }
-            __syncthreads();
-            uint32_t hi_bin, lo_bin, rest2;
-            pick_bin(rhist, 512, false, krem, hi_bin, rest2, nullptr);
-            for (int i = tid; i < 256; i += SEL_THREADS) rhist[i] = 0;
-            __syncthreads();
-            for (uint32_t i0 = 0; i0 < n_cand; i0 += SEL_THREADS) {
-                const uint32_t i = i0 + tid;
-                const unsigned long long c = i < n_cand ? cand[i] : 0ull;
-                const uint32_t pos = ~(uint32_t)c;
-                hist_add(rhist, i < n_cand && (uint32_t)(c >> 32) == thr && (pos >> 8) == hi_bin, pos & 255u);
-            }
-            __syncthreads();
-            pick_bin(rhist, 256, false, rest2, lo_bin, rest2, nullptr);
-            const uint32_t idx_max = (hi_bin << 8) | lo_bin;         // largest position taken among the ties
-            // ---- surviving candidates fill the threshold bin's range of the staging buffer
-            for (uint32_t i0 = 0; i0 < n_cand; i0 += SEL_THREADS) {
-                const uint32_t i = i0 + tid;
-                const unsigned long long c = i < n_cand ? cand[i] : 0ull;
-                const uint32_t key = (uint32_t)(c >> 32), pos = ~(uint32_t)c;
-                const bool take = i < n_cand && (key > thr || (key == thr && pos <= idx_max));
-                const unsigned long long m = __ballot(take);
-                if (m != 0ull) {
-                    uint32_t bs = 0;
-                    const int first = __ffsll((long long)m) - 1;
-                    if (lane == first) bs = atomicAdd(&sh_nsurv, (uint32_t)__popcll(m));
-                    bs = __shfl(bs, first) + (uint32_t)__popcll(m & ((1ull << lane) - 1ull));
-                    if (take && base0 + bs < (uint32_t)LI_MAX_SELECT) stage[base0 + bs] = c;
-                }
-            }
-            if (tid == 0) atomicMax(&sh_longest, rest);              // this range is ordered like the others
-        }
+    // ---- 3. bucket of every candidate of the wave's own region (up to eight per lane) and its slot
+    // inside the bucket
+    constexpr int CPT = SEL_WAVE_CAP / 64;
+    unsigned long long ce[CPT];
+    uint32_t cb[CPT], cslot[CPT];
+#pragma unroll
+    for (int u = 0; u < CPT; ++u) {
+        const uint32_t j = (uint32_t)(u * 64 + lane);
+        const unsigned long long raw = cand[wv * SEL_WAVE_CAP + (j < wave_count ? j : 0u)];
+        ce[u] = j < wave_count ? order_word(__uint_as_float((uint32_t)raw), (uint32_t)(raw >> 32)) : 0ull;
+    }
+#pragma unroll
+    for (int u = 0; u < CPT; ++u) {
+        const uint32_t lin = (uint32_t)fmaxf((key_score((uint32_t)(ce[u] >> 32)) - blo) * bscale, 0.f);
+        cb[u] = (uint32_t)SEL_BUCKETS - 1u - (lin < (uint32_t)SEL_BUCKETS ? lin : (uint32_t)SEL_BUCKETS - 1u);
+        cslot[u] = 0u;
+        if ((uint32_t)(u * 64 + lane) < wave_count) cslot[u] = atomicAdd(&bcount[cb[u]], 1u);
+    }
+    __syncthreads();
+    uint32_t n_cand = 0;
+#pragma unroll
+    for (int i = 0; i < SEL_WAVES; ++i) n_cand += wave_tot[i];
+    if (sh_over != 0u || n_cand < (uint32_t)k) {
+        __syncthreads();                                         // wave_tot is reused below
+        select_streaming(p, t, hist, stage);                     // uniform: the whole workgroup goes
+        return;
+    }
+
+    // ---- 4. bucket offsets (two buckets per thread) and the bucket holding the k-th best key
+    {
+        const uint32_t b0 = 2u * (uint32_t)tid;
+        const uint32_t c0 = bcount[b0], c1 = bcount[b0 + 1u];
+        const uint32_t tot = c0 + c1;
+        const uint32_t incl = wave_incl_scan(tot);
+        __syncthreads();                                         // every wave has read the candidate counts
+        if (lane == 63) wave_tot[wv] = incl;
         __syncthreads();
-        const bool direct = n_cand <= (uint32_t)SEL_DIRECT_MAX;      // threshold range already in sortbuf
-        const uint32_t n_stage = direct ? base0 : (uint32_t)k;       // entries of stage[] to order
-        if (sh_longest > (uint32_t)SEL_RANK_MAX) {
-            // a long range: sort everything at once
-            int width = 64;
-            while (width < k) width <<= 1;
-            for (int i = tid; i < width; i += SEL_THREADS) {
-                unsigned long long e = 0ull;
-                if ((uint32_t)i < n_stage) e = stage[i];
-                else if (i < k) e = sortbuf[i];
-                cand[i] = e;
-            }
-            __syncthreads();
-            bitonic_sort_desc(cand, width, tid);
-            for (int i = tid; i < k; i += SEL_THREADS) sortbuf[i] = cand[i];
-            __syncthreads();
-        } else {
-            // ---- order every bin's range by counting
-            for (uint32_t i = tid; i < n_stage; i += SEL_THREADS) {
-                const unsigned long long e = stage[i];
-                const uint32_t kb = (uint32_t)(e >> (64 - HIST_BITS));
-                const uint32_t cnt = kb == bin0 ? rest : hist[kb];
-                const uint32_t end = kb == bin0 ? (uint32_t)k : cursor[kb];
-                const uint32_t beg = end - cnt;
-                sortbuf[beg + count_greater(stage, beg, end, e)] = e;
-            }
-            __syncthreads();
+        uint32_t before = incl - tot;
+#pragma unroll
+        for (int i = 0; i < SEL_WAVES; ++i) before += i < wv ? wave_tot[i] : 0u;
+        boff[b0] = before;
+        boff[b0 + 1u] = before + c0;
+        if (before < (uint32_t)k && (uint32_t)k <= before + c0) sh_tb = b0;
+        else if (before + c0 < (uint32_t)k && (uint32_t)k <= before + tot) sh_tb = b0 + 1u;
+    }
+    __syncthreads();
+    const uint32_t tb = sh_tb;
+    const uint32_t n_stage = boff[tb] + bcount[tb];
+    if (n_stage > (uint32_t)SEL_STAGE) {
+        __syncthreads();
+        select_streaming(p, t, hist, stage);
+        return;
+    }
+#pragma unroll
+    for (int u = 0; u < CPT; ++u) {
+        if ((uint32_t)(u * 64 + lane) < wave_count && cb[u] <= tb) {
+            const uint32_t idx = boff[cb[u]] + cslot[u];
+            stage[idx] = ce[u];
+            sbucket[idx] = (uint16_t)cb[u];
         }
     }
-    for (int i = tid; i < k; i += SEL_THREADS)
-        out[i] = i < nsel ? (int32_t)(~(uint32_t)(sortbuf[i] & 0xffffffffull)) : -1;
+    __syncthreads();
+    // Order inside buckets by counting.  Neighbouring threads take neighbouring staged entries, which
+    // mostly share a bucket, so the loop lengths of a wave agree and its LDS reads are broadcasts; a
+    // thread's two entries are ranked side by side, four keys of each bucket per trip, to keep eight
+    // reads in flight.  Entries past the first 2048 (the tail of the last bucket) take a second trip
+    // that only the waves holding them make.
+    for (uint32_t i0 = 0; i0 < n_stage; i0 += 2 * SEL_THREADS) {
+        if (i0 + (uint32_t)(wv * 64) >= n_stage) break;          // wave-uniform: nothing staged for this wave
+        unsigned long long e[2];
+        uint32_t beg[2], len[2], rank[2];
+        uint32_t maxlen = 0;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t i = i0 + (uint32_t)(q * SEL_THREADS + tid);
+            const bool ok = i < n_stage;
+            e[q] = stage[ok ? i : 0u];
+            const uint32_t bk = sbucket[ok ? i : 0u];
+            beg[q] = boff[bk];
+            len[q] = ok ? bcount[bk] : 0u;
+            rank[q] = 0u;
+            maxlen = len[q] > maxlen ? len[q] : maxlen;
+        }
+        for (uint32_t j = 0; j < maxlen; j += 4) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+#pragma unroll
+                for (uint32_t d = 0; d < 4; ++d) {
+                    const bool in = j + d < len[q];
+                    const unsigned long long x = stage[in ? beg[q] + j + d : 0u];
+                    rank[q] += (in && x > e[q]) ? 1u : 0u;
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t fin = beg[q] + rank[q];
+            if (i0 + (uint32_t)(q * SEL_THREADS + tid) < n_stage && fin < (uint32_t)k) out[fin] = (int32_t)(~(uint32_t)e[q]);
+        }
+    }
 }
 
 __global__ __launch_bounds__(SEL_THREADS) void li_select_stream_kernel(const LiParams p)
