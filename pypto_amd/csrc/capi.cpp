@@ -219,10 +219,10 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.q_dt = a->q_scale_dtype;
     p.k_dt = a->k_scale_dtype;
     p.w_dt = a->weight_dtype;
-    {   // enough waves to cover every SIMD a few times, at most 8 blocks (256 keys) per wave
-        const long long blocks = (long long)a->t * ((p.score_stride + 31) / 32);
-        long long bpw = blocks / ((long long)cu_count() * 4 * 4);
-        p.bpw = (int)(bpw < 1 ? 1 : (bpw > 8 ? 8 : bpw));
+    {   // enough waves to cover every SIMD a few times, at most 8 pairs (512 keys) per wave
+        const long long pairs = (long long)a->t * ((p.score_stride + 63) / 64);
+        long long ppw = pairs / ((long long)cu_count() * 4 * 4);
+        p.ppw = (int)(ppw < 1 ? 1 : (ppw > 8 ? 8 : ppw));
     }
     hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));

@@ -23,7 +23,7 @@ struct LiParams {
     long long score_stride;
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes
-    int bpw;                // 32-key blocks per wave of the score kernel
+    int ppw;                // 64-key block pairs per wave of the score kernel
 };
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream);

@@ -11,10 +11,12 @@
 //
 // Kernels
 //   li_score_kernel   w_scale[h] = fp16(q_scale * weight) if both fp16, else the fp32 product;
-//                     one wave per run of 32-key blocks: v_mfma_i32_32x32x32_i8 with A = the
+//                     one wave per run of 64-key pairs of blocks: v_mfma_i32_32x32x32_i8 with A = the
 //                     token's 64 query heads (two 32-row operands resident in registers) and
-//                     B = 32 key rows loaded straight from the paged cache in operand layout;
-//                     epilogue in registers; scores to a [T, max_seq] fp32 workspace
+//                     B = 32 key rows loaded straight from the paged cache in operand layout; a
+//                     half-wave swap gives every lane all 64 heads of one key, summed in registers
+//                     with the per-head factors in scalar registers; scores to a [T, max_seq] fp32
+//                     workspace
 //   li_select_kernel  one workgroup per query token, keys ordered by the strict word
 //                     (score image << 32 | ~position): a histogram of a 2048-score sample gives a
 //                     pivot, one pass over the row compacts the keys above it, those are spread over
@@ -45,13 +47,6 @@ __device__ __forceinline__ float load_scalar(const void *p, size_t i, int dt)
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
-// relu, scale by 2^-11, round to fp16, back to fp32
-__device__ __forceinline__ float relu_fp16_term(const int dot)
-{
-    const float r = (float)(dot > 0 ? dot : 0) * (1.0f / 2048.0f);
-    return (float)(_Float16)r;
-}
-
 // w_scale[h] = fp16(q_scale * weight) when both are fp16 (one fp16 rounding of the exact product),
 // else the fp32 product
 __device__ __forceinline__ float w_scale_of(const LiParams &p, const size_t i)
@@ -71,9 +66,60 @@ __device__ __forceinline__ uint32_t score_key(const float x)
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-__global__ __launch_bounds__(256) void li_score_kernel(const LiParams p)
+// fp32 product of one half of a packed fp16 pair with a wave-uniform fp32 factor, rounded once:
+// v_fma_mix_f32 widens the fp16 operand on the fly.  The addend +0 turns a product of -0 into +0, which
+// no later step can tell apart: the running sum starts at +0 and so never is -0 itself.
+template <int HI>
+__device__ __forceinline__ float mul_f16_f32(const uint32_t packed, const float w)
 {
-    __shared__ float wsh[4][LI_HEADS];
+    float r;
+    if (HI)
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "s"(w));
+    else
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "s"(w));
+    return r;
+}
+
+// x = fp16(relu(dot) / 2048) for two dots, packed.  v_fma_mixlo/mixhi_f16 scale in fp32 (exact: a power
+// of two) and round once to fp16; -|dot|/2048 rounds to a negative fp16 that the packed integer max
+// then clears, which equals clearing first.  scale = 2^-11 in a scalar register.
+__device__ __forceinline__ uint32_t relu_fp16_pair(const int d0, const int d1, const float scale)
+{
+    uint32_t packed;
+    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(packed) : "v"((float)d0), "s"(scale));
+    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(packed) : "v"((float)d1), "s"(scale));
+    // relu on the bit patterns: a negative fp16 (and -0) is a negative 16-bit integer
+    typedef __attribute__((ext_vector_type(2))) short s16x2;
+    const s16x2 zero = {0, 0};
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2, packed), zero));
+}
+
+constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // one staged pair of 32-key blocks
+
+// One wave scores runs of 64 consecutive keys: two 32-key blocks X and Y per trip.
+//   stage  key rows travel from the paged cache into the wave's own LDS buffers with
+//          global_load_lds: consecutive lanes fetch consecutive 16-byte chunks, so every request is a
+//          run of whole cache lines (loading the operand layout directly touches 32 lines with 32
+//          bytes each per instruction and is bound by the address unit).  Chunk c of row r lands at
+//          position c ^ (r & 7) of the row, which makes the operand reads below conflict-free.  The
+//          pair after the current one is in flight while the current one is scored.
+//   MFMA   A = the token's 64 query heads as two 32-row operands (resident in registers), B = 32 key
+//          rows read from LDS in operand layout; four accumulators per trip.  With the head
+//          permutation below, lane (j, half) of block X's accumulators holds heads 32*half ..
+//          32*half + 31 of key X_j, likewise for Y.
+//   swap   after relu / scale / fp16 packing, v_permlane32_swap exchanges the upper half-wave of X's
+//          registers with the lower half-wave of Y's: lane j < 32 then holds all 64 heads of key X_j
+//          and lane 32 + j all 64 heads of key Y_j, the same head in the same register on every lane.
+//   sum    every lane runs the sequential head sum h = 0..63 of its own key; the per-head factors are
+//          wave-uniform and sit in scalar registers.
+// At least two waves per SIMD: the 256 registers that leaves per lane are all architectural, so the
+// matrix instructions accumulate in ordinary vector registers and the epilogue reads them directly.
+// KDT = dtype code of the key scales: a compile-time choice keeps the scale load free of branches, so
+// it stays in flight beside the staged rows.
+template <int KDT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void li_score_kernel(const LiParams p)
+{
+    __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_PAIR_BYTES];
     const int t = blockIdx.y;
     const int b = t / p.S1;
     int cur = p.act[b];
@@ -83,16 +129,62 @@ __global__ __launch_bounds__(256) void li_score_kernel(const LiParams p)
     const int l = threadIdx.x & 63;
     const int j = l & 31;
     const int half = l >> 5;
-    const int key0 = (blockIdx.x * 4 + w) * (p.bpw * 32);
+    const int key0 = (blockIdx.x * 4 + w) * (p.ppw * 64);
     if (key0 >= cur) return;
-    int nblk = (cur - key0 + 31) >> 5;
-    nblk = nblk > p.bpw ? p.bpw : nblk;
+    int npair = (cur - key0 + 63) >> 6;
+    npair = npair > p.ppw ? p.ppw : npair;
+    const int last_blk = ((cur + 31) >> 5) - 1;                  // last 32-key block holding a valid key
+
+    // First cache row of every 32-key block of this wave's run, looked up once: lane i holds the row of
+    // block i of the run (32 consecutive positions never straddle a page; a run has at most 16 blocks;
+    // blocks past the end of the sequence repeat the last valid block).
+    int run_row;
+    {
+        int blk = (key0 >> 5) + (l & 15);
+        blk = blk > last_blk ? last_blk : blk;
+        const int pos0 = 32 * blk;
+        const int page = pos0 / p.bs;
+        int pb = p.bt[(size_t)b * p.maxblk + page];
+        pb = pb < 0 ? 0 : (pb >= p.nblocks ? p.nblocks - 1 : pb);
+        run_row = pb * p.bs + (pos0 - page * p.bs);
+    }
+    // Requests pair pr into buffer buf: per block four instructions of eight rows each.  Lane l owns
+    // LDS slot l of an instruction's 1 KiB, i.e. row l/8 and position l%8, and fetches chunk
+    // (l%8) ^ (l/8) of that row; the instruction offset moves the cache address and the LDS address
+    // alike.  Written as assembly so that the requests stay outstanding until the explicit wait at the
+    // top of the trip that consumes them.  ksc = the scale of the key whose sum this lane will hold
+    // (X_j on the lower half-wave, Y_j on the upper).
+    const uint32_t lane_off = (uint32_t)((l >> 3) * LI_DIM + (((l & 7) ^ (l >> 3)) << 4));
+    const uint32_t lds_base = (uint32_t)__builtin_amdgcn_readfirstlane(
+        (int)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t *)&kstage[w][0][0]);
+    auto request_pair = [&](const int pr, const int buf, float &ksc) {
+        const int rx = __builtin_amdgcn_readlane(run_row, 2 * pr), ry = __builtin_amdgcn_readlane(run_row, 2 * pr + 1);
+        const int8_t *gx = p.kcache + (size_t)rx * LI_DIM;
+        const int8_t *gy = p.kcache + (size_t)ry * LI_DIM;
+        const uint32_t dst = lds_base + (uint32_t)(buf * SC_PAIR_BYTES);
+        asm volatile("s_mov_b32 m0, %2\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dwordx4 %0, %1\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:3072"
+                     :: "v"(lane_off), "s"(gx), "s"(dst) : "memory", "m0");
+        asm volatile("s_mov_b32 m0, %2\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dwordx4 %0, %1\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+                     "global_load_lds_dwordx4 %0, %1 offset:3072"
+                     :: "v"(lane_off), "s"(gy), "s"(dst + 4096u) : "memory", "m0");
+        ksc = load_scalar(p.k_scale, (size_t)(half ? ry : rx) + j, KDT);
+    };
+    float ksa, ksb;
+    request_pair(0, 0, ksa);
 
     // A operands.  Row i of operand 0 is head 32*((i>>2)&1) + 4*(i>>3) + (i&3), operand 1 adds 16:
     // with the 32x32 accumulator layout (row = 8*(r/4) + 4*half + r%4) lane (key, half) then holds
     // heads 32*half + r in register r of accumulator 0 and heads 32*half + 16 + r in accumulator 1.
-    // The contraction is taken in the order bytes [64*half + 16*ks, +16) so that a lane's four key
-    // loads are one contiguous 64-byte run.
+    // The contraction runs over 16-byte chunks in the order 4*half + ks (ks = 0..3).
     i32x4 qa[2][4];
     {
         const int head0 = 32 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3);
@@ -103,72 +195,79 @@ __global__ __launch_bounds__(256) void li_score_kernel(const LiParams p)
             qa[1][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * LI_DIM + 16 * ks);
         }
     }
-    // per-head factors: lane l computes head l's, the wave shares them through its LDS slice
-    float wsc[32];
+    // per-head factors: lane l computes head l's; read back lane by lane they are wave-uniform
+    float wsc[LI_HEADS];
     {
-        wsh[w][l] = w_scale_of(p, (size_t)t * LI_HEADS + l);
-        const f32x4 *src = reinterpret_cast<const f32x4 *>(&wsh[w][32 * half]);
+        const float mine = w_scale_of(p, (size_t)t * LI_HEADS + l);
 #pragma unroll
-        for (int r4 = 0; r4 < 8; ++r4) {
-            const f32x4 v = src[r4];
-            wsc[4 * r4] = v[0]; wsc[4 * r4 + 1] = v[1]; wsc[4 * r4 + 2] = v[2]; wsc[4 * r4 + 3] = v[3];
-        }
-    }
-
-    // key rows of block blk of this wave: 32 consecutive positions never straddle a page
-    auto block_row = [&](const int blk) -> size_t {
-        const int pos0 = key0 + 32 * blk;
-        const int page = pos0 / p.bs;
-        int pb = p.bt[(size_t)b * p.maxblk + page];
-        pb = pb < 0 ? 0 : (pb >= p.nblocks ? p.nblocks - 1 : pb);
-        return (size_t)pb * p.bs + (pos0 - page * p.bs) + j;
-    };
-    i32x4 kf[4], kn[4];
-    float ksc, kscn;
-    {
-        const size_t row = block_row(0);
-        const int8_t *kp = p.kcache + row * LI_DIM + 64 * half;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) kf[ks] = *reinterpret_cast<const i32x4 *>(kp + 16 * ks);
-        ksc = load_scalar(p.k_scale, row, p.k_dt);
+        for (int h = 0; h < LI_HEADS; ++h) wsc[h] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), h));
     }
 
     float *srow = p.scores + (size_t)t * p.score_stride;
-    for (int blk = 0; blk < nblk; ++blk) {
-        {   // next block's rows are in flight while this one is scored (the last iteration reloads itself)
-            const size_t row = block_row(blk + 1 < nblk ? blk + 1 : blk);
-            const int8_t *kp = p.kcache + row * LI_DIM + 64 * half;
+    // 2^-11 as a run-time value, so that it sits in a scalar register (the mix instructions take no literal)
+    const float scale = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3a000000));
+    // this lane's operand chunks of row j inside a staged block
+    int koff[4];
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) kn[ks] = *reinterpret_cast<const i32x4 *>(kp + 16 * ks);
-            kscn = load_scalar(p.k_scale, row, p.k_dt);
-        }
-        i32x16 acc0, acc1;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { acc0[r] = 0; acc1[r] = 0; }
+    for (int ks = 0; ks < 4; ++ks) koff[ks] = j * LI_DIM + (((4 * half + ks) ^ (j & 7)) << 4);
+
+    // one trip: the operands of the staged pair are read, the following pair is requested into the
+    // other buffer, then the pair is scored
+    auto trip = [&](const int pr, const int buf, const float ksc, float &kscn) {
+        const int8_t *src = &kstage[w][buf][0];
+        i32x4 kx[4], ky[4];
+        __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0): the staged pair has landed
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[0][ks], kf[ks], acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[1][ks], kf[ks], acc1, 0, 0, 0);
+            kx[ks] = *reinterpret_cast<const i32x4 *>(src + koff[ks]);
+            ky[ks] = *reinterpret_cast<const i32x4 *>(src + 4096 + koff[ks]);
         }
-        float prod[32];
+        if (pr + 1 < npair) request_pair(pr + 1, buf ^ 1, kscn);
+        i32x16 ax0, ax1, ay0, ay1;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            prod[r] = __fmul_rn(wsc[r], relu_fp16_term(acc0[r]));
-            prod[16 + r] = __fmul_rn(wsc[16 + r], relu_fp16_term(acc1[r]));
+        for (int r = 0; r < 16; ++r) { ax0[r] = 0; ax1[r] = 0; ay0[r] = 0; ay1[r] = 0; }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            ax0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[0][ks], kx[ks], ax0, 0, 0, 0);
+            ax1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[1][ks], kx[ks], ax1, 0, 0, 0);
+            ay0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[0][ks], ky[ks], ay0, 0, 0, 0);
+            ay1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[1][ks], ky[ks], ay1, 0, 0, 0);
         }
-        // heads 0..31 are summed by the lower half-wave, whose partial sum then seeds heads 32..63
-        // in the upper half-wave: the chain is the sequential sum h = 0..63.
-        float lo = 0.f;
+        // lo[o][i] / hi[o][i]: heads 16*o + 2*i, +1 (lo) and 32 + 16*o + 2*i, +1 (hi) of this lane's key
+        uint32_t lo[2][8], hi[2][8];
 #pragma unroll
-        for (int r = 0; r < 32; ++r) lo = __fadd_rn(lo, prod[r]);
-        float hi = __shfl(lo, j);
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t x0 = relu_fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale), y0 = relu_fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale);
+            const uint32_t x1 = relu_fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale), y1 = relu_fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale);
+            const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+            lo[0][i] = s0[0]; hi[0][i] = s0[1];
+            lo[1][i] = s1[0]; hi[1][i] = s1[1];
+        }
+        float sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 32; ++r) hi = __fadd_rn(hi, prod[r]);
-        const int pos = key0 + 32 * blk + j;
-        if (half == 1 && pos < cur) srow[pos] = __fmul_rn(hi, ksc);
+        for (int o = 0; o < 2; ++o) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) kf[ks] = kn[ks];
-        ksc = kscn;
+            for (int i = 0; i < 8; ++i) {
+                sum = __fadd_rn(sum, mul_f16_f32<0>(lo[o][i], wsc[16 * o + 2 * i]));
+                sum = __fadd_rn(sum, mul_f16_f32<1>(lo[o][i], wsc[16 * o + 2 * i + 1]));
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < 2; ++o) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                sum = __fadd_rn(sum, mul_f16_f32<0>(hi[o][i], wsc[32 + 16 * o + 2 * i]));
+                sum = __fadd_rn(sum, mul_f16_f32<1>(hi[o][i], wsc[32 + 16 * o + 2 * i + 1]));
+            }
+        }
+        const int pos = key0 + 64 * pr + l;
+        if (pos < cur) srow[pos] = __fmul_rn(sum, ksc);
+    };
+    for (int pr = 0; pr < npair; pr += 2) {
+        trip(pr, 0, ksa, ksb);
+        if (pr + 1 < npair) trip(pr + 1, 1, ksb, ksa);
     }
 }
 
@@ -780,8 +879,11 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_stream_kernel(const LiP
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream)
 {
-    const unsigned gx = (unsigned)((p.score_stride + 4 * p.bpw * 32 - 1) / (4 * p.bpw * 32));
-    hipLaunchKernelGGL(li_score_kernel, dim3(gx, (unsigned)p.T), dim3(256), 0, stream, p);
+    const unsigned gx = (unsigned)((p.score_stride + 4 * p.ppw * 64 - 1) / (4 * p.ppw * 64));
+    const dim3 grid(gx, (unsigned)p.T), block(256);
+    if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
+    else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP16>, grid, block, 0, stream, p);
+    else hipLaunchKernelGGL(li_score_kernel<PTO_DT_BF16>, grid, block, 0, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(li_select_kernel, dim3((unsigned)p.T), dim3(SEL_THREADS), 0, stream, p);
