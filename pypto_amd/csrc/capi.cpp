@@ -219,10 +219,11 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.q_dt = a->q_scale_dtype;
     p.k_dt = a->k_scale_dtype;
     p.w_dt = a->weight_dtype;
-    {   // enough waves to cover every SIMD a few times, at most 8 pairs (512 keys) per wave
+    {   // A wave pays three dependent memory latencies before its first pair, so runs are made as long
+        // as still leaves every SIMD two rounds of two waves; at most 32 pairs (2048 keys) per wave.
         const long long pairs = (long long)a->t * ((p.score_stride + 63) / 64);
         long long ppw = pairs / ((long long)cu_count() * 4 * 4);
-        p.ppw = (int)(ppw < 1 ? 1 : (ppw > 8 ? 8 : ppw));
+        p.ppw = (int)(ppw < 1 ? 1 : (ppw > pto::LI_MAX_PAIRS_PER_WAVE ? pto::LI_MAX_PAIRS_PER_WAVE : ppw));
     }
     hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));

@@ -9,6 +9,7 @@ constexpr int LI_MAX_SELECT = 2048;     // most indices one query token can rece
 constexpr int LI_MAX_SEQ = 128 * 1024;  // longest key sequence
 constexpr int LI_HEADS = 64;
 constexpr int LI_DIM = 128;
+constexpr int LI_MAX_PAIRS_PER_WAVE = 32;  // a wave keeps one cache-row index per 32-key block of its run in a lane
 
 struct LiParams {
     const int8_t *q;        // [T, 64, 128]
@@ -23,7 +24,7 @@ struct LiParams {
     long long score_stride;
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes
-    int ppw;                // 64-key block pairs per wave of the score kernel
+    int ppw;                // 64-key block pairs per wave of the score kernel, <= LI_MAX_PAIRS_PER_WAVE
 };
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream);

@@ -94,7 +94,8 @@ __device__ __forceinline__ uint32_t relu_fp16_pair(const int d0, const int d1, c
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2, packed), zero));
 }
 
-constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // one staged pair of 32-key blocks
+constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // key rows of one staged pair of 32-key blocks
+constexpr int SC_BUF_BYTES = SC_PAIR_BYTES + 256;   // + the 64 key scales (one dword per lane)
 
 // One wave scores runs of 64 consecutive keys: two 32-key blocks X and Y per trip.
 //   stage  key rows travel from the paged cache into the wave's own LDS buffers with
@@ -119,7 +120,7 @@ constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // one staged pair of 32-key bloc
 template <int KDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void li_score_kernel(const LiParams p)
 {
-    __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_PAIR_BYTES];
+    __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_BUF_BYTES];
     const int t = blockIdx.y;
     const int b = t / p.S1;
     int cur = p.act[b];
@@ -136,11 +137,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
     const int last_blk = ((cur + 31) >> 5) - 1;                  // last 32-key block holding a valid key
 
     // First cache row of every 32-key block of this wave's run, looked up once: lane i holds the row of
-    // block i of the run (32 consecutive positions never straddle a page; a run has at most 16 blocks;
+    // block i of the run (32 consecutive positions never straddle a page; a run has at most 64 blocks;
     // blocks past the end of the sequence repeat the last valid block).
     int run_row;
     {
-        int blk = (key0 >> 5) + (l & 15);
+        int blk = (key0 >> 5) + l;
         blk = blk > last_blk ? last_blk : blk;
         const int pos0 = 32 * blk;
         const int page = pos0 / p.bs;
@@ -151,17 +152,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
     // Requests pair pr into buffer buf: per block four instructions of eight rows each.  Lane l owns
     // LDS slot l of an instruction's 1 KiB, i.e. row l/8 and position l%8, and fetches chunk
     // (l%8) ^ (l/8) of that row; the instruction offset moves the cache address and the LDS address
-    // alike.  Written as assembly so that the requests stay outstanding until the explicit wait at the
-    // top of the trip that consumes them.  ksc = the scale of the key whose sum this lane will hold
-    // (X_j on the lower half-wave, Y_j on the upper).
+    // alike.  A ninth instruction stages the dword holding the scale of the key whose sum this lane
+    // will hold (X_j on the lower half-wave, Y_j on the upper).  Every load of the loop is written as
+    // assembly: the compiler then tracks none of them, and the explicit waits of the trips decide
+    // alone how long requests stay outstanding (two pairs ahead).
     const uint32_t lane_off = (uint32_t)((l >> 3) * LI_DIM + (((l & 7) ^ (l >> 3)) << 4));
     const uint32_t lds_base = (uint32_t)__builtin_amdgcn_readfirstlane(
         (int)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t *)&kstage[w][0][0]);
-    auto request_pair = [&](const int pr, const int buf, float &ksc) {
+    constexpr int KSZ = KDT == PTO_DT_FP32 ? 4 : 2;
+    auto request_pair = [&](const int pr, const int buf) {
         const int rx = __builtin_amdgcn_readlane(run_row, 2 * pr), ry = __builtin_amdgcn_readlane(run_row, 2 * pr + 1);
         const int8_t *gx = p.kcache + (size_t)rx * LI_DIM;
         const int8_t *gy = p.kcache + (size_t)ry * LI_DIM;
-        const uint32_t dst = lds_base + (uint32_t)(buf * SC_PAIR_BYTES);
+        const uint32_t dst = lds_base + (uint32_t)(buf * SC_BUF_BYTES);
         asm volatile("s_mov_b32 m0, %2\n\t"
                      "s_nop 0\n\t"
                      "global_load_lds_dwordx4 %0, %1\n\t"
@@ -176,10 +179,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
                      "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
                      "global_load_lds_dwordx4 %0, %1 offset:3072"
                      :: "v"(lane_off), "s"(gy), "s"(dst + 4096u) : "memory", "m0");
-        ksc = load_scalar(p.k_scale, (size_t)(half ? ry : rx) + j, KDT);
+        // the aligned dword that holds this lane's scale
+        const uintptr_t sa = (reinterpret_cast<uintptr_t>(p.k_scale) + ((size_t)(half ? ry : rx) + j) * KSZ) & ~(uintptr_t)3;
+        asm volatile("s_mov_b32 m0, %1\n\t"
+                     "s_nop 0\n\t"
+                     "global_load_lds_dword %0, off"
+                     :: "v"(sa), "s"(dst + (uint32_t)SC_PAIR_BYTES) : "memory", "m0");
     };
-    float ksa, ksb;
-    request_pair(0, 0, ksa);
+    request_pair(0, 0);
+    if (npair > 1) request_pair(1, 1);
 
     // A operands.  Row i of operand 0 is head 32*((i>>2)&1) + 4*(i>>3) + (i&3), operand 1 adds 16:
     // with the 32x32 accumulator layout (row = 8*(r/4) + 4*half + r%4) lane (key, half) then holds
@@ -211,19 +219,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) koff[ks] = j * LI_DIM + (((4 * half + ks) ^ (j & 7)) << 4);
 
-    // one trip: the operands of the staged pair are read, the following pair is requested into the
-    // other buffer, then the pair is scored
-    auto trip = [&](const int pr, const int buf, const float ksc, float &kscn) {
+    // One trip.  Requests complete in the order they were made, so "at most nine outstanding" (the
+    // nine of the following pair; the score store of the previous trip may or may not be among them)
+    // means that this trip's pair has landed.  Its operands and scale move to registers, which frees
+    // the buffer for the pair two ahead; then the pair is scored.
+    auto trip = [&](const int pr, const int buf) {
         const int8_t *src = &kstage[w][buf][0];
         i32x4 kx[4], ky[4];
-        __builtin_amdgcn_s_waitcnt(0x0F70);                      // vmcnt(0): the staged pair has landed
+        if (pr + 1 < npair) __builtin_amdgcn_s_waitcnt(0x0F79);  // vmcnt(9)
+        else __builtin_amdgcn_s_waitcnt(0x0F70);                 // vmcnt(0)
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             kx[ks] = *reinterpret_cast<const i32x4 *>(src + koff[ks]);
             ky[ks] = *reinterpret_cast<const i32x4 *>(src + 4096 + koff[ks]);
         }
-        if (pr + 1 < npair) request_pair(pr + 1, buf ^ 1, kscn);
+        const uint32_t ksraw = *reinterpret_cast<const uint32_t *>(src + SC_PAIR_BYTES + 4 * l);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): the buffer has been read
+        if (pr + 2 < npair) request_pair(pr + 2, buf);
+        float ksc;
+        if (KDT == PTO_DT_FP32) {
+            ksc = __uint_as_float(ksraw);
+        } else {
+            // rows of a block are 32 consecutive scales, so the parity of the lane's element follows j
+            const int rrow = __builtin_amdgcn_readlane(run_row, 2 * pr + 0);
+            const int rrow1 = __builtin_amdgcn_readlane(run_row, 2 * pr + 1);
+            const bool odd = ((reinterpret_cast<uintptr_t>(p.k_scale) + ((size_t)(half ? rrow1 : rrow) + j) * KSZ) & 2) != 0;
+            const uint16_t hbits = (uint16_t)(odd ? ksraw >> 16 : ksraw);
+            ksc = KDT == PTO_DT_BF16 ? bf16_bits_to_f32(hbits) : (float)__builtin_bit_cast(_Float16, hbits);
+        }
         i32x16 ax0, ax1, ay0, ay1;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { ax0[r] = 0; ax1[r] = 0; ay0[r] = 0; ay1[r] = 0; }
@@ -266,8 +291,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
         if (pos < cur) srow[pos] = __fmul_rn(sum, ksc);
     };
     for (int pr = 0; pr < npair; pr += 2) {
-        trip(pr, 0, ksa, ksb);
-        if (pr + 1 < npair) trip(pr + 1, 1, ksb, ksa);
+        trip(pr, 0);
+        if (pr + 1 < npair) trip(pr + 1, 1);
     }
 }
 
