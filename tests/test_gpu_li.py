@@ -79,3 +79,51 @@ def test_config1_full_size(c_oracle):
     for variant in ("fp16", "fp32"):
         inp = gen_indexer_inputs(4, 1, [32768] * 4, selected_count=2048, seed=1, variant=variant)
         assert_exact(run_op(inp), oracle(inp, c_oracle), f"cfg1 {variant}")
+
+
+def test_bf16_key_scales(c_oracle):
+    """Key scales in bf16 (two per staged dword, either half), fp16 query scales, bf16 weights."""
+    inp = gen_indexer_inputs(2, 2, [4500, 2600], selected_count=2048, seed=51, variant="fp32")
+    inp.idx_key_scale = inp.idx_key_scale.to(torch.bfloat16)
+    inp.idx_query_scale = inp.idx_query_scale.to(torch.float16)
+    assert_exact(run_op(inp), oracle(inp, c_oracle), "bf16 key scales")
+
+
+def test_long_runs_wide_block_table(c_oracle):
+    """64 query tokens over a block table 1024 pages wide: the launch then gives every wave the longest
+    run of keys it supports, the lengths end inside runs, pairs and 32-key blocks, and the longest
+    sequence is the maximum the operator accepts (131072)."""
+    from pypto_amd.synthetic import gen_block_table
+    g = torch.Generator().manual_seed(61)
+    act = [131072, 65536 + 17, 40000, 2049, 2048, 2047, 4096 + 33, 1] + \
+          [int(x) for x in torch.randint(1, 3000, [56], generator=g)]
+    block_num, table = gen_block_table(act, 128, g, shuffle=True, max_kv=131072)
+    inp = gen_indexer_inputs(len(act), 1, act, selected_count=2048, seed=62, variant="fp32", block_table=table,
+                             block_num=block_num)
+    assert_exact(run_op(inp), oracle(inp, c_oracle), "wide block table")
+
+
+def test_small_pages_and_small_k(c_oracle):
+    """32-key pages (every block of a pair on its own page) and small selection counts."""
+    for k, act in ((1, [5000, 70]), (17, [2500, 31]), (512, [700, 513])):
+        inp = gen_indexer_inputs(2, 1, act, selected_count=k, seed=70 + k, variant="fp16", block_size=32)
+        assert_exact(run_op(inp), oracle(inp, c_oracle), f"bs=32 k={k}")
+
+
+def test_select_falls_back_on_degenerate_rows(c_oracle):
+    """Rows the sampled pivot cannot split: a constant row with one spike (every sampled score equal),
+    and two-valued scores where far more than the list holds tie above the pivot."""
+    inp = gen_indexer_inputs(2, 1, [40000, 30000], selected_count=2048, seed=81, variant="fp32")
+    kc = inp.idx_key_cache.reshape(-1, 128)
+    ks = inp.idx_key_scale.reshape(-1)
+    pos0 = torch.arange(40000)
+    phys0 = inp.block_table[0].long()[pos0 // 128] * 128 + pos0 % 128
+    kc[phys0] = kc[phys0[0]].clone()              # token 0: every key equal ...
+    ks[phys0] = ks[phys0[0]].clone()
+    ks[phys0[12345]] = ks[phys0[0]].clone() * 4   # ... except one, four times the score
+    pos1 = torch.arange(30000)
+    phys1 = inp.block_table[1].long()[pos1 // 128] * 128 + pos1 % 128
+    kc[phys1] = kc[phys1[0]].clone()              # token 1: two score values, 3/4 of the keys on the larger
+    ks[phys1] = ks[phys1[0]].clone()
+    ks[phys1[pos1 % 4 == 1]] = ks[phys1[0]].clone() * 0.5
+    assert_exact(run_op(inp), oracle(inp, c_oracle), "degenerate rows")
