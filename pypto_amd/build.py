@@ -23,7 +23,7 @@ HIPCC_FLAGS = [
     "-ffp-contract=on",
     # packed fp32 arithmetic is switched off for all device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm",
 ]
 
 

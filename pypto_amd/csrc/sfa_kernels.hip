@@ -439,6 +439,437 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     }
 }
 
+// ------------------------------------------------------------------ pipelined kernel, 128 heads
+//
+// Same decomposition and numerics as sfa_decode_kernel<4>, re-scheduled so that the matrix cores, the
+// LDS and the vector ALU work at the same time.  Per tile n every wave runs two phases:
+//   A  S(n+1) = K(n+1) . Q^T        (36 matrix products)  with the de-quantisation of tile n+2
+//   B  O^T   += V(n)^T . P(n)^T     (32 matrix products)  with the softmax of S(n+1)
+// and one barrier.  Tiles travel  cache --(LDS-DMA, four tiles ahead)--> int8 staging  --(phase A,
+// two tiles ahead)--> bf16 tile --> phase A (K) and, one iteration later, phase B (V).  A wave
+// stages and de-quantises the same eight keys of every tile, so the staging buffers need no barrier;
+// the rope part of a row is bf16 already and is requested straight into the buffer phase A reads.
+//
+// LDS (bytes):  3 bf16 tiles of 32 x 520 (nope part; 1040 B pitch)      99840
+//               4 rope buffers of 32 x 64 bf16 (16-byte chunk c of key k at position c ^ (k & 7))
+//               2 int8 staging buffers of 32 x 512, 2 x 32 x 4 fp32 scales
+//               row table of the split (logical position -> cache row)
+// The prologue borrows the tile area to stage Q^T in two passes of 288 contraction dims
+// (592 B pitch per head: 36 chunks + 1 pad, which spreads eight heads over all banks).
+namespace pl {
+constexpr int NPITCH = DN + 8;                                     // tile row pitch in elements
+constexpr int TILE_BYTES = KT * NPITCH * 2;                        // 33280
+constexpr int ROPE_BYTES = KT * DR * 2;                            // 4096
+constexpr int STG_BYTES = KT * DN;                                 // 16384
+constexpr int SC_BYTES = KT * 16;                                  // 512
+constexpr int OFF_TILE = 0;
+constexpr int OFF_ROPE = OFF_TILE + 3 * TILE_BYTES;
+constexpr int OFF_STG = OFF_ROPE + 4 * ROPE_BYTES;
+constexpr int OFF_SC = OFF_STG + 2 * STG_BYTES;
+constexpr int OFF_ROWS = OFF_SC + 2 * SC_BYTES;
+constexpr int LDS_BYTES = OFF_ROWS + (SFA_MAX_CHUNK + KT) * 4;     // 158336
+constexpr int QCHUNKS = 36;                                        // 16-byte chunks per head and pass
+constexpr int QPITCH = (QCHUNKS + 1) * 16;                         // 592
+constexpr int QINSTR = (32 * (QCHUNKS + 1) + 63) / 64;             // 19 requests of 1 KiB per wave and pass
+constexpr int QREGION = QINSTR * 1024;
+static_assert(4 * QREGION <= 3 * TILE_BYTES, "Q staging must fit in the tile area");
+static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+}  // namespace pl
+
+typedef __attribute__((address_space(3))) uint8_t lds_byte_t;
+
+// One LDS-DMA request: lane i's 16 bytes at gaddr land at lds_dst + 16*i.  lds_dst is wave-uniform.
+// Written as assembly so that the compiler tracks none of these requests: the explicit vmcnt waits of
+// the kernel decide how long they stay outstanding.
+__device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
+}
+// the same for lanes 0..7 only (128 bytes)
+__device__ __forceinline__ void dma16_low8(const void *gaddr, const uint32_t lds_dst)
+{
+    uint64_t saved;
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    asm volatile("s_mov_b64 %0, exec\n\t"
+                 "s_mov_b64 exec, 0xff\n\t"
+                 "s_mov_b32 m0, %2\n\t"
+                 "s_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, off\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(gaddr), "s"(dst)
+                 : "memory", "m0");
+}
+
+__global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaParams p)
+{
+    using namespace pl;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
+    int *const rows_lds = reinterpret_cast<int *>(lds + OFF_ROWS);
+
+    const int tid = threadIdx.x;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l = tid & 63;
+    const int half = l >> 5;
+    const int col = l & 31;
+    const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_byte_t *)lds);
+
+    // workgroups of one query row share an XCD (consecutive workgroup ids rotate over the 8 XCDs)
+    const int per_row = p.hgroups * p.nsplit;
+    const int xcd = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    const int t = (slot / per_row) * 8 + xcd;
+    if (t >= p.T) return;
+    const int within = slot % per_row;
+    const int hg = within / p.nsplit;
+    const int sp = within % p.nsplit;
+    const int b = t / p.S1;
+    const int s1i = t - b * p.S1;
+
+    int cur = p.act[b] - p.S1 + 1 + s1i;
+    cur = cur < 0 ? 0 : (cur > p.topk ? p.topk : cur);
+    const int ntile = (cur + KT - 1) / KT;
+    const int tiles_per_split = (ntile + p.nsplit - 1) / p.nsplit;
+    const int k_begin = sp * tiles_per_split * KT;
+    int k_end = k_begin + tiles_per_split * KT;
+    k_end = k_end > cur ? cur : k_end;
+    const int n_valid = k_end > k_begin ? k_end - k_begin : 0;
+    const int nt = (n_valid + KT - 1) / KT;                     // tiles of this split
+
+    const int head = hg * 128 + w * 32 + col;
+    const bool head_ok = head < p.NQ;
+
+    // ---- row table first: its loads must not queue behind the bulk requests below.  Keys past k_end
+    // in the last tile repeat the split's first key (finite data, masked out of the softmax).
+    for (int i = tid; i < nt * KT; i += 256) {
+        const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
+        int blk = idx / p.bs;
+        blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
+        long long row = (long long)p.bt[(size_t)b * p.maxblk + blk] * p.bs + (idx - (idx / p.bs) * p.bs);
+        row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
+        rows_lds[i] = (int)row;
+    }
+    __syncthreads();
+
+    // requests this wave's eight keys of tile m: rope (one request), scales (lanes 0..7), nope (four)
+    auto request_tile = [&](const int m) {
+        const int *rt = rows_lds + m * KT + 8 * w;
+        {
+            const int kk = l >> 3;
+            dma16(p.kr + (size_t)rt[kk] * DR + 8 * ((l & 7) ^ kk), lds0 + OFF_ROPE + (m & 3) * ROPE_BYTES + w * 1024);
+        }
+        dma16_low8(p.ksc + (size_t)rt[l & 7] * 4, lds0 + OFF_SC + (m & 1) * SC_BYTES + w * 128);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            dma16(p.kn + (size_t)rt[2 * i + half] * DN + 16 * col, lds0 + OFF_STG + (m & 1) * STG_BYTES + w * (8 * DN) + i * 1024);
+    };
+    // De-quantisation of key kk (0..7) of this wave's share of tile m into tile buffer tb, in two
+    // halves: the staged bytes and the scale are read one step before they are converted, so that no
+    // step waits for its own LDS reads.
+    u32x2 dq_raw;
+    float dq_sc;
+    auto dequant_read = [&](const int m, const int kk) {
+        const int key = 8 * w + kk;
+        dq_raw = *reinterpret_cast<const u32x2 *>(lds + OFF_STG + (m & 1) * STG_BYTES + key * DN + 8 * l);
+        dq_sc = *reinterpret_cast<const float *>(lds + OFF_SC + (m & 1) * SC_BYTES + key * 16 + 4 * (l >> 4));
+    };
+    auto dequant_write = [&](const int tb, const int kk) {
+        const int key = 8 * w + kk;
+        dequant8((int)dq_raw[0], (int)dq_raw[1], dq_sc, reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb * TILE_BYTES) + key * NPITCH + 8 * l);
+    };
+    auto dequant_key = [&](const int m, const int tb, const int kk) {
+        dequant_read(m, kk);
+        dequant_write(tb, kk);
+    };
+
+    if (nt > 0) request_tile(0);
+    if (nt > 1) request_tile(1);
+
+    // ---- Q^T fragments: lane (head, half) holds q[head][16*ks + 8*half .. +8], staged per wave (its own
+    // 32 heads) in two passes.  Slot s of a pass is chunk s % 37 of head s / 37 (chunk 36 is padding);
+    // heads past NQ read the last head and are never stored.
+    bf16x8 qf[KSTEPS];
+    {
+        const uint32_t qdst = lds0 + OFF_TILE + w * QREGION;
+        const uint8_t *qsrc = lds + OFF_TILE + w * QREGION + col * QPITCH + 16 * half;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll 1
+            for (int i = 0; i < QINSTR; ++i) {
+                const int sl = i * 64 + l;
+                int hl = sl / (QCHUNKS + 1);
+                int c = sl - hl * (QCHUNKS + 1);
+                hl = hl > 31 ? 31 : hl;
+                c = c >= QCHUNKS ? 0 : c;
+                int hd = hg * 128 + w * 32 + hl;
+                hd = hd < p.NQ ? hd : p.NQ - 1;
+                const size_t qrow = (size_t)t * p.NQ + hd;
+                const int dim = pass * (8 * QCHUNKS) + 8 * c;         // first of the chunk's 8 contraction dims
+                const uint16_t *src = dim < DN ? p.q_nope + qrow * DN + dim : p.q_rope + qrow * DR + (dim - DN);
+                dma16(src, qdst + i * 1024);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0)
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS / 2; ++ks) qf[pass * (KSTEPS / 2) + ks] = *reinterpret_cast<const bf16x8 *>(qsrc + 32 * ks);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xC07F);                       // lgkmcnt(0): the region may be overwritten
+        }
+    }
+    __syncthreads();                                                  // the tile area is free
+
+    f32x16 o[DVB];
+#pragma unroll
+    for (int i = 0; i < DVB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+    valu_to_mfma_fence();
+    float m_run = -INFINITY;   // reference max, log2 domain
+    float l_run = 0.f;         // running sum of exp2(s - m_run)
+
+    // Issue order.  A wave issues in order and a matrix product occupies the matrix pipe for 32 cycles,
+    // so the next product in program order stalls everything behind it: vector and LDS instructions
+    // overlap with the matrix pipe only when they sit BETWEEN two products, about seven of them at
+    // most.  Both phases are therefore written as "slots" -- one product, the operand reads of a later
+    // product, one small piece of vector work -- and a scheduling barrier after every slot keeps the
+    // compiler from regrouping them.
+
+    // S^T of tile buffer tb / rope buffer rb: 36 slots; micro(ks) is the caller's piece of vector work.
+    // Operand reads stay four products ahead.
+    auto gemm1 = [&](const int tb, const int rb, f32x16 &s, auto &&micro) {
+        const uint16_t *arow = reinterpret_cast<const uint16_t *>(lds + OFF_TILE + tb * TILE_BYTES) + col * NPITCH + 8 * half;
+        const uint8_t *rrow = lds + OFF_ROPE + rb * ROPE_BYTES + col * (DR * 2);
+        bf16x8 fa[2][4];
+        auto read_a = [&](const int ks) -> bf16x8 {
+            return ks < DN / 16 ? *reinterpret_cast<const bf16x8 *>(arow + 16 * ks)
+                                : *reinterpret_cast<const bf16x8 *>(rrow + (((2 * (ks - DN / 16) + half) ^ (col & 7)) << 4));
+        };
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fa[0][e] = read_a(e);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[(ks >> 2) & 1][ks & 3], qf[ks], s, 0, 0, 0);
+            if (ks + 4 < KSTEPS) fa[((ks >> 2) + 1) & 1][ks & 3] = read_a(ks + 4);
+            micro(ks);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Online softmax of the S^T block in s (already masked and still unscaled), cut into 32 slots that
+    // ride between the matrix products of the PV phase.  Lane (head, half) holds keys
+    // kt + 8*(r/4) + 4*half + r%4.  The reference max follows the true max lazily: probabilities may
+    // reach 2^RESCALE_TAU, which fp32 sums and bf16 P hold without loss, and the accumulators are
+    // rescaled (by the caller, before the tile's PV products) only on a jump.  A tile entirely past
+    // k_end leaves the running state as it is: every probability is exp2(-inf) = 0.
+    float sm_mx = 0.f, sm_mnew = 0.f, sm_alpha = 1.0f, sm_lsum = 0.f;
+    bool sm_rescale = false;
+    auto softmax_micro = [&](const int m, f32x16 &s, bf16x8 (&pf)[2]) {
+        if (m < 4) {                                            // scale
+#pragma unroll
+            for (int r = 4 * m; r < 4 * m + 4; ++r) s[r] *= p.scale_log2;
+        } else if (m < 8) {                                     // running max
+            const int r = 4 * (m - 4);
+            const float part = fmaxf(fmaxf(s[r], s[r + 1]), fmaxf(s[r + 2], s[r + 3]));
+            sm_mx = m == 4 ? part : fmaxf(sm_mx, part);
+        } else if (m == 8) {                                    // both half-waves, then the lazy reference
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(sm_mx), __float_as_uint(sm_mx), false, false);
+            sm_mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+            const bool upd = sm_mx > m_run + RESCALE_TAU;       // always true on the first tile (m_run = -inf)
+            sm_mnew = upd ? sm_mx : m_run;
+            sm_rescale = upd && l_run > 0.f;                    // nothing accumulated yet: nothing to rescale
+        } else if (m == 9) {
+            sm_alpha = sm_mnew > m_run ? __builtin_amdgcn_exp2f(m_run - sm_mnew) : 1.0f;
+        } else if (m < 26) {                                    // one exponential per slot
+            const int r = m - 10;
+            s[r] = __builtin_amdgcn_exp2f(s[r] - sm_mnew);
+        } else if (m < 28) {                                    // row sum
+            const int r = 8 * (m - 26);
+            const float part = ((s[r] + s[r + 1]) + (s[r + 2] + s[r + 3])) + ((s[r + 4] + s[r + 5]) + (s[r + 6] + s[r + 7]));
+            sm_lsum = m == 26 ? part : sm_lsum + part;
+        } else if (m == 28) {
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(sm_lsum), __float_as_uint(sm_lsum), false, false);
+            sm_lsum = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            l_run = l_run * sm_alpha + sm_lsum;
+            m_run = sm_mnew;
+        } else if (m < 31) {                                    // P^T fragments
+            const int kk = m - 29;
+            u32x4 pk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = pack_bf16x2(s[8 * kk + 2 * e], s[8 * kk + 2 * e + 1]);
+            pf[kk] = __builtin_bit_cast(bf16x8, pk);
+        }
+    };
+    // keys past k_end of the tile starting at kt
+    auto mask_tail = [&](const int kt, f32x16 &s) {
+        if (kt + KT > k_end) {                   // only the split's last tile (or a tile past it)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (kt + 8 * (r >> 2) + 4 * half + (r & 3) >= k_end) s[r] = -INFINITY;
+        }
+    };
+
+    // ---- pipeline fill: tiles 0 and 1 de-quantised, tiles 2 and 3 requested, S(0) and its softmax
+    f32x16 s;
+    bf16x8 pf_cur[2], pf_next[2];
+    if (nt > 0) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) dequant_key(0, 0, kk);
+        if (nt > 1) {
+#pragma unroll
+            for (int kk = 0; kk < 8; ++kk) dequant_key(1, 1, kk);
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (nt > 2) request_tile(2);
+        if (nt > 3) request_tile(3);
+        __syncthreads();
+        gemm1(0, 0, s, [](int) {});
+        mask_tail(k_begin, s);
+#pragma unroll
+        for (int m = 0; m < 32; ++m) softmax_micro(m, s, pf_cur);
+        sm_rescale = false;
+    }
+
+    int tb_cur = 0;                          // tile buffer of tile n: n % 3
+    for (int n = 0; n < nt; ++n) {
+        const int tb_next = tb_cur == 2 ? 0 : tb_cur + 1;
+        const int tb_fill = tb_next == 2 ? 0 : tb_next + 1;
+
+        // ---- phase A: S(n+1) with the de-quantisation of this wave's keys of tile n+2 (one key per
+        // group of four products), then the request for tile n+4 into the staging buffer just read.
+        // Past the last tile the products run on stale data; the softmax below masks all of it.
+        if (n + 3 < nt) __builtin_amdgcn_s_waitcnt(0x0F76);      // vmcnt(6): tile n+2 staged, n+3 may be in flight
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+        dequant_read(n + 2, 0);
+        {
+            u32x2 raw;
+            float sc, bias;
+            u32x4 outv;
+            uint32_t v = 0;
+            gemm1(tb_next, (n + 1) & 3, s, [&](const int ks) {
+                const int g = ks >> 2, e = ks & 3;               // key g of the wave's eight, quarter e of its 8 values
+                if (g >= 8) return;
+                if (e == 0) {
+                    raw = dq_raw;
+                    sc = dq_sc;
+                    if (g + 1 < 8) dequant_read(n + 2, g + 1);
+                    bias = -128.0f * sc;
+                }
+                if ((e & 1) == 0) v = raw[e >> 1] ^ 0x80808080u;
+                // same arithmetic as dequant8: fma(float(byte + 128), sc, -128*sc) rounds x*sc once
+                const float f0 = __builtin_fmaf((float)((v >> (16 * (e & 1))) & 0xffu), sc, bias);
+                const float f1 = __builtin_fmaf((float)((v >> (16 * (e & 1) + 8)) & 0xffu), sc, bias);
+                outv[e] = pack_bf16x2(f0, f1);
+                if (e == 3)
+                    *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb_fill * TILE_BYTES) +
+                                               (8 * w + g) * NPITCH + 8 * l) = outv;
+            });
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): the staging buffer has been read
+        if (n + 4 < nt) request_tile(n + 4);
+
+        // ---- phase B: O^T += V(n)^T . P(n)^T, product m = 16*kk + dvb, with the softmax of S(n+1)
+        if (__any(sm_rescale)) {             // a jump of the reference max found by the softmax of S(n)
+            mfma_to_valu_fence();
+            AccLoop<0, DVB>::scale(o, sm_alpha);
+            valu_to_mfma_fence();
+        }
+        {
+            const int kt_next = k_begin + (n + 1) * KT;
+            const uint16_t *vbase = reinterpret_cast<const uint16_t *>(lds + OFF_TILE + tb_cur * TILE_BYTES) +
+                                    (4 * half + ((l & 15) >> 2)) * NPITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+            s16x4 va[2][4][2];
+            auto read_v = [&](const int m, s16x4 (&v)[2]) {     // V^T operand of product m
+                const uint16_t *a0 = vbase + (16 * (m >> 4)) * NPITCH + 32 * (m & 15);
+                v[0] = lds_read_tr16(a0);
+                v[1] = lds_read_tr16(a0 + 8 * NPITCH);
+            };
+#pragma unroll
+            for (int e = 0; e < 4; ++e) read_v(e, va[0][e]);
+            mask_tail(kt_next, s);
+#pragma unroll
+            for (int m = 0; m < 32; ++m) {
+                const s16x8 a = __builtin_shufflevector(va[(m >> 2) & 1][m & 3][0], va[(m >> 2) & 1][m & 3][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf_cur[m >> 4]);
+                if (m + 4 < 32) read_v(m + 4, va[((m >> 2) + 1) & 1][m & 3]);
+                softmax_micro(m, s, pf_next);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+        pf_cur[0] = pf_next[0];
+        pf_cur[1] = pf_next[1];
+        tb_cur = tb_next;
+    }
+
+    // ---- epilogue: as in sfa_decode_kernel (transposition through per-wave slices of the tile area)
+    mfma_to_valu_fence();
+    {
+        float *stage = reinterpret_cast<float *>(lds) + w * (32 * 128);
+        float *inv_tab = reinterpret_cast<float *>(rows_lds) + w * 32;      // the row table is dead by now
+        const int head_base = hg * 128 + w * 32;
+        const size_t prow_base = ((size_t)t * p.nsplit + sp) * p.NQ;
+        if (half == 0) inv_tab[col] = l_run > 0.f ? 1.0f / l_run : 0.f;
+        auto drain = [&](auto final_tag, auto all_tag) {
+            constexpr bool FINAL = decltype(final_tag)::value;
+            constexpr bool ALL = decltype(all_tag)::value;
+            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 4 * col
+                                   : p.part_o + (prow_base + head_base + half) * DN + 4 * col;
+#pragma unroll
+            for (int gq = 0; gq < DVB / 4; ++gq) {
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const f32x16 &acc = o[4 * gq + b4];
+                        const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
+                        *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
+                    }
+#pragma unroll 1
+                for (int pq = 0; pq < 2; ++pq) {
+                    f32x4 rv[8];
+                    float iv[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int hl = 2 * (8 * pq + e) + half;
+                        rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
+                        iv[e] = inv_tab[hl];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int hl = 2 * (8 * pq + e) + half;
+                        const f32x4 v = rv[e] * iv[e];
+                        u32x2 pk;
+                        pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
+                        pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
+                        if (ALL || head_base + hl < p.NQ)
+                            *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN + 128 * gq) = pk;
+                    }
+                }
+            }
+        };
+        const bool all_heads = head_base + 32 <= p.NQ;
+        if (p.nsplit == 1) {
+            if (all_heads) drain(std::true_type{}, std::true_type{});
+            else drain(std::true_type{}, std::false_type{});
+        } else {
+            if (all_heads) drain(std::false_type{}, std::true_type{});
+            else drain(std::false_type{}, std::false_type{});
+        }
+        if (p.nsplit > 1 && half == 0 && head_ok) {
+            p.part_ml[(prow_base + head) * 2] = m_run;
+            p.part_ml[(prow_base + head) * 2 + 1] = l_run;
+        }
+    }
+}
+
 // Merges the key splits of one query row: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - m)
 // and O_s the split's normalised fp16 partial.  One thread per (row, head, 8 value channels).
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
@@ -484,7 +915,7 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
     switch (p.waves) {
     case 1: hipLaunchKernelGGL(sfa_decode_kernel<1>, dim3(grid), dim3(64), 0, stream, p); break;
     case 2: hipLaunchKernelGGL(sfa_decode_kernel<2>, dim3(grid), dim3(128), 0, stream, p); break;
-    default: hipLaunchKernelGGL(sfa_decode_kernel<4>, dim3(grid), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL(sfa_decode_pipelined_kernel, dim3(grid), dim3(256), 0, stream, p); break;
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
