@@ -445,7 +445,10 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 // LDS and the vector ALU work at the same time.  Per tile n every wave runs two phases:
 //   A  S(n+1) = K(n+1) . Q^T        (36 matrix products)  with the de-quantisation of tile n+2
 //   B  O^T   += V(n)^T . P(n)^T     (32 matrix products)  with the softmax of S(n+1)
-// and one barrier.  Tiles travel  cache --(LDS-DMA, four tiles ahead)--> int8 staging  --(phase A,
+// with a barrier after each.  For the first product a wave owns 32 heads (Q^T fragments in registers,
+// the whole K tile read from LDS); for the second it owns 128 value channels of ALL 128 heads, so it
+// reads only its quarter of V^T and takes P^T -- 8 KiB per tile, exchanged through LDS -- as the
+// other operand.  That halves the LDS traffic of the second product, which is what bounds the loop.  Tiles travel  cache --(LDS-DMA, four tiles ahead)--> int8 staging  --(phase A,
 // two tiles ahead)--> bf16 tile --> phase A (K) and, one iteration later, phase B (V).  A wave
 // stages and de-quantises the same eight keys of every tile, so the staging buffers need no barrier;
 // the rope part of a row is bf16 already and is requested straight into the buffer phase A reads.
@@ -453,7 +456,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 // LDS (bytes):  3 bf16 tiles of 32 x 520 (nope part; 1040 B pitch)      99840
 //               4 rope buffers of 32 x 64 bf16 (16-byte chunk c of key k at position c ^ (k & 7))
 //               2 int8 staging buffers of 32 x 512, 2 x 32 x 4 fp32 scales
-//               row table of the split (logical position -> cache row)
+//               P^T of the current tile, per-head rescale factors
+//               row table of the split (logical position -> cache row), at most 1024 keys
 // The prologue borrows the tile area to stage Q^T in two passes of 288 contraction dims
 // (592 B pitch per head: 36 chunks + 1 pad, which spreads eight heads over all banks).
 namespace pl {
@@ -466,8 +470,11 @@ constexpr int OFF_TILE = 0;
 constexpr int OFF_ROPE = OFF_TILE + 3 * TILE_BYTES;
 constexpr int OFF_STG = OFF_ROPE + 4 * ROPE_BYTES;
 constexpr int OFF_SC = OFF_STG + 2 * STG_BYTES;
-constexpr int OFF_ROWS = OFF_SC + 2 * SC_BYTES;
-constexpr int LDS_BYTES = OFF_ROWS + (SFA_MAX_CHUNK + KT) * 4;     // 158336
+constexpr int P_BYTES = 2 * 2 * 128 * 16;                          // P^T of one tile: [16-key step][half][head] x 16 B
+constexpr int OFF_P = OFF_SC + 2 * SC_BYTES;
+constexpr int OFF_ALPHA = OFF_P + P_BYTES;                         // 128 rescale factors (later 1/l), 2 flags
+constexpr int OFF_ROWS = OFF_ALPHA + 128 * 4 + 16;
+constexpr int LDS_BYTES = OFF_ROWS + (SFA_PIPE_MAX_CHUNK + KT) * 4;
 constexpr int QCHUNKS = 36;                                        // 16-byte chunks per head and pass
 constexpr int QPITCH = (QCHUNKS + 1) * 16;                         // 592
 constexpr int QINSTR = (32 * (QCHUNKS + 1) + 63) / 64;             // 19 requests of 1 KiB per wave and pass
@@ -735,13 +742,25 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         sm_rescale = false;
     }
 
+    float *const alpha_tab = reinterpret_cast<float *>(lds + OFF_ALPHA);
+    int *const resc_flag = reinterpret_cast<int *>(lds + OFF_ALPHA + 128 * 4);
+    if (tid < 2) resc_flag[tid] = 0;
+
     int tb_cur = 0;                          // tile buffer of tile n: n % 3
     for (int n = 0; n < nt; ++n) {
         const int tb_next = tb_cur == 2 ? 0 : tb_cur + 1;
         const int tb_fill = tb_next == 2 ? 0 : tb_next + 1;
 
+        // P(n)^T and the rescale factors found by the softmax of S(n) go to LDS for all waves
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+            *reinterpret_cast<bf16x8 *>(lds + OFF_P + (((kk * 2 + half) * 128 + 32 * w + col) << 4)) = pf_cur[kk];
+        if (half == 0) alpha_tab[32 * w + col] = sm_alpha;
+        if (__any(sm_rescale) && l == 0) resc_flag[n & 1] = 1;
+        if (tid == 0) resc_flag[(n + 1) & 1] = 0;
+
         // ---- phase A: S(n+1) with the de-quantisation of this wave's keys of tile n+2 (one key per
-        // group of four products), then the request for tile n+4 into the staging buffer just read.
+        // four products), then the request for tile n+4 into the staging buffer just read.
         // Past the last tile the products run on stale data; the softmax below masks all of it.
         if (n + 3 < nt) __builtin_amdgcn_s_waitcnt(0x0F76);      // vmcnt(6): tile n+2 staged, n+3 may be in flight
         else __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -774,31 +793,44 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): the staging buffer has been read
         if (n + 4 < nt) request_tile(n + 4);
+        __syncthreads();
 
-        // ---- phase B: O^T += V(n)^T . P(n)^T, product m = 16*kk + dvb, with the softmax of S(n+1)
-        if (__any(sm_rescale)) {             // a jump of the reference max found by the softmax of S(n)
+        // ---- phase B: O^T[128 channels of this wave][128 heads] += V(n)^T . P(n)^T with the softmax of
+        // S(n+1).  Product m = 16*kk + 4*i + hb: 16-key step kk, channel block i, head block hb.
+        if (__builtin_amdgcn_readfirstlane(resc_flag[n & 1]) != 0) {   // some head's reference max jumped
+            float al[4];
+#pragma unroll
+            for (int hb = 0; hb < 4; ++hb) al[hb] = alpha_tab[32 * hb + col];
             mfma_to_valu_fence();
-            AccLoop<0, DVB>::scale(o, sm_alpha);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int hb = 0; hb < 4; ++hb) acc_scale(o[4 * i + hb], al[hb]);
             valu_to_mfma_fence();
         }
         {
             const int kt_next = k_begin + (n + 1) * KT;
             const uint16_t *vbase = reinterpret_cast<const uint16_t *>(lds + OFF_TILE + tb_cur * TILE_BYTES) +
-                                    (4 * half + ((l & 15) >> 2)) * NPITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
-            s16x4 va[2][4][2];
-            auto read_v = [&](const int m, s16x4 (&v)[2]) {     // V^T operand of product m
-                const uint16_t *a0 = vbase + (16 * (m >> 4)) * NPITCH + 32 * (m & 15);
+                                    (4 * half + ((l & 15) >> 2)) * NPITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3) + 128 * w;
+            const uint8_t *pbase = lds + OFF_P + ((half * 128 + col) << 4);
+            bf16x8 bq[2][4];
+            s16x4 av[2][2];
+            auto read_v = [&](const int m, s16x4 (&v)[2]) {     // V^T operand of products m .. m+3
+                const uint16_t *a0 = vbase + (16 * (m >> 4)) * NPITCH + 32 * ((m >> 2) & 3);
                 v[0] = lds_read_tr16(a0);
                 v[1] = lds_read_tr16(a0 + 8 * NPITCH);
             };
 #pragma unroll
-            for (int e = 0; e < 4; ++e) read_v(e, va[0][e]);
+            for (int hb = 0; hb < 4; ++hb) bq[0][hb] = *reinterpret_cast<const bf16x8 *>(pbase + ((32 * hb) << 4));
+            read_v(0, av[0]);
             mask_tail(kt_next, s);
 #pragma unroll
             for (int m = 0; m < 32; ++m) {
-                const s16x8 a = __builtin_shufflevector(va[(m >> 2) & 1][m & 3][0], va[(m >> 2) & 1][m & 3][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf_cur[m >> 4]);
-                if (m + 4 < 32) read_v(m + 4, va[((m >> 2) + 1) & 1][m & 3]);
+                const int kk = m >> 4, i = (m >> 2) & 3, hb = m & 3;
+                const s16x8 a = __builtin_shufflevector(av[(m >> 2) & 1][0], av[(m >> 2) & 1][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                acc_mfma(o[4 * i + hb], __builtin_bit_cast(bf16x8, a), bq[kk][hb]);
+                if (hb == 0 && m + 4 < 32) read_v(m + 4, av[((m >> 2) + 1) & 1]);
+                if (m < 4) bq[1][m] = *reinterpret_cast<const bf16x8 *>(pbase + ((2 * 128 + 32 * m) << 4));
                 softmax_micro(m, s, pf_next);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -809,60 +841,74 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         tb_cur = tb_next;
     }
 
-    // ---- epilogue: as in sfa_decode_kernel (transposition through per-wave slices of the tile area)
+    // ---- epilogue.  Wave w holds value channels 128*w .. +127 of all 128 heads: accumulator
+    // o[4*i + hb], lane (head, half) = channels 128*w + 32*i + 8*(r/4) + 4*half + r%4 of head 32*hb + head.
+    // One head block at a time goes through the wave's slice of the (now idle) tile area, 32 heads x
+    // 128 channels fp32 with 16-byte chunk c of head h at chunk c ^ (h & 7), so that 32 lanes write
+    // 256 contiguous bytes of one head.  The 1/l factors of all heads are shared through LDS.
     mfma_to_valu_fence();
     {
         float *stage = reinterpret_cast<float *>(lds) + w * (32 * 128);
-        float *inv_tab = reinterpret_cast<float *>(rows_lds) + w * 32;      // the row table is dead by now
-        const int head_base = hg * 128 + w * 32;
+        float *inv_tab = alpha_tab;
         const size_t prow_base = ((size_t)t * p.nsplit + sp) * p.NQ;
-        if (half == 0) inv_tab[col] = l_run > 0.f ? 1.0f / l_run : 0.f;
-        auto drain = [&](auto final_tag, auto all_tag) {
+        if (half == 0) inv_tab[32 * w + col] = l_run > 0.f ? 1.0f / l_run : 0.f;
+        __syncthreads();
+        // FINAL: bf16 result rows; otherwise fp16 partial of a key split (O / l of the split, merged by
+        // the combine kernel with weights l * 2^(m - m_max); O / l is a convex combination of
+        // de-quantised V rows, so it stays finite in fp16 as long as |int8 * scale| < 65504).
+        // ALL: every head of the block exists, so the stores need no predicate.  Both are uniform and
+        // resolved outside the loops: scalar branches inside them cost more than the work.
+        auto drain = [&](auto hb_tag, auto final_tag, auto all_tag) {
+            constexpr int HB = decltype(hb_tag)::value;
             constexpr bool FINAL = decltype(final_tag)::value;
             constexpr bool ALL = decltype(all_tag)::value;
-            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 4 * col
-                                   : p.part_o + (prow_base + head_base + half) * DN + 4 * col;
+            const int head_base = hg * 128 + 32 * HB;
+            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 128 * w + 4 * col
+                                   : p.part_o + (prow_base + head_base + half) * DN + 128 * w + 4 * col;
 #pragma unroll
-            for (int gq = 0; gq < DVB / 4; ++gq) {
+            for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
-                for (int b4 = 0; b4 < 4; ++b4)
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        const f32x16 &acc = o[4 * gq + b4];
-                        const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
-                        *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
-                    }
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const f32x16 &acc = o[4 * b4 + HB];
+                    const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
+                    *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
+                }
 #pragma unroll 1
-                for (int pq = 0; pq < 2; ++pq) {
-                    f32x4 rv[8];
-                    float iv[8];
+            for (int pq = 0; pq < 2; ++pq) {
+                f32x4 rv[8];
+                float iv[8];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int hl = 2 * (8 * pq + e) + half;
-                        rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
-                        iv[e] = inv_tab[hl];
-                    }
+                for (int e = 0; e < 8; ++e) {
+                    const int hl = 2 * (8 * pq + e) + half;
+                    rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
+                    iv[e] = inv_tab[32 * HB + hl];
+                }
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int hl = 2 * (8 * pq + e) + half;
-                        const f32x4 v = rv[e] * iv[e];
-                        u32x2 pk;
-                        pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
-                        pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
-                        if (ALL || head_base + hl < p.NQ)
-                            *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN + 128 * gq) = pk;
-                    }
+                for (int e = 0; e < 8; ++e) {
+                    const int hl = 2 * (8 * pq + e) + half;
+                    const f32x4 v = rv[e] * iv[e];
+                    u32x2 pk;
+                    pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
+                    pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
+                    if (ALL || head_base + hl < p.NQ)
+                        *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN) = pk;
                 }
             }
         };
-        const bool all_heads = head_base + 32 <= p.NQ;
-        if (p.nsplit == 1) {
-            if (all_heads) drain(std::true_type{}, std::true_type{});
-            else drain(std::true_type{}, std::false_type{});
-        } else {
-            if (all_heads) drain(std::false_type{}, std::true_type{});
-            else drain(std::false_type{}, std::false_type{});
-        }
+        auto drain_block = [&](auto hb_tag) {
+            const bool all_heads = hg * 128 + 32 * decltype(hb_tag)::value + 32 <= p.NQ;
+            if (p.nsplit == 1) {
+                if (all_heads) drain(hb_tag, std::true_type{}, std::true_type{});
+                else drain(hb_tag, std::true_type{}, std::false_type{});
+            } else {
+                if (all_heads) drain(hb_tag, std::false_type{}, std::true_type{});
+                else drain(hb_tag, std::false_type{}, std::false_type{});
+            }
+        };
+        drain_block(std::integral_constant<int, 0>{});
+        drain_block(std::integral_constant<int, 1>{});
+        drain_block(std::integral_constant<int, 2>{});
+        drain_block(std::integral_constant<int, 3>{});
         if (p.nsplit > 1 && half == 0 && head_ok) {
             p.part_ml[(prow_base + head) * 2] = m_run;
             p.part_ml[(prow_base + head) * 2 + 1] = l_run;
