@@ -458,8 +458,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 //               2 int8 staging buffers of 32 x 512, 2 x 32 x 4 fp32 scales
 //               P^T of the current tile, per-head rescale factors
 //               row table of the split (logical position -> cache row), at most 1024 keys
-// The prologue borrows the tile area to stage Q^T in two passes of 288 contraction dims
-// (592 B pitch per head: 36 chunks + 1 pad, which spreads eight heads over all banks).
+// The prologue borrows the tile area to stage Q^T in two passes (nope dims 0..255, then 256..511 and
+// the rope dims), every head row with its 16-byte chunks XOR-swizzled by the head number.
 namespace pl {
 constexpr int NPITCH = DN + 8;                                     // tile row pitch in elements
 constexpr int TILE_BYTES = KT * NPITCH * 2;                        // 33280
@@ -475,10 +475,7 @@ constexpr int OFF_P = OFF_SC + 2 * SC_BYTES;
 constexpr int OFF_ALPHA = OFF_P + P_BYTES;                         // 128 rescale factors (later 1/l), 2 flags
 constexpr int OFF_ROWS = OFF_ALPHA + 128 * 4 + 16;
 constexpr int LDS_BYTES = OFF_ROWS + (SFA_PIPE_MAX_CHUNK + KT) * 4;
-constexpr int QCHUNKS = 36;                                        // 16-byte chunks per head and pass
-constexpr int QPITCH = (QCHUNKS + 1) * 16;                         // 592
-constexpr int QINSTR = (32 * (QCHUNKS + 1) + 63) / 64;             // 19 requests of 1 KiB per wave and pass
-constexpr int QREGION = QINSTR * 1024;
+constexpr int QREGION = 20 * 1024;                                 // Q^T staging per wave: 16 KiB nope half + 4 KiB rope
 static_assert(4 * QREGION <= 3 * TILE_BYTES, "Q staging must fit in the tile area");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 }  // namespace pl
@@ -492,6 +489,12 @@ __device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
 {
     const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
+}
+// the same with a wave-uniform base address and a 32-bit byte offset per lane
+__device__ __forceinline__ void dma16_base(const void *base, const uint32_t lane_off, const uint32_t lds_dst)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory", "m0");
 }
 // the same for lanes 0..7 only (128 bytes)
 __device__ __forceinline__ void dma16_low8(const void *gaddr, const uint32_t lds_dst)
@@ -547,18 +550,6 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
     const int head = hg * 128 + w * 32 + col;
     const bool head_ok = head < p.NQ;
 
-    // ---- row table first: its loads must not queue behind the bulk requests below.  Keys past k_end
-    // in the last tile repeat the split's first key (finite data, masked out of the softmax).
-    for (int i = tid; i < nt * KT; i += 256) {
-        const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
-        int blk = idx / p.bs;
-        blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
-        long long row = (long long)p.bt[(size_t)b * p.maxblk + blk] * p.bs + (idx - (idx / p.bs) * p.bs);
-        row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
-        rows_lds[i] = (int)row;
-    }
-    __syncthreads();
-
     // requests this wave's eight keys of tile m: rope (one request), scales (lanes 0..7), nope (four)
     auto request_tile = [&](const int m) {
         const int *rt = rows_lds + m * KT + 8 * w;
@@ -581,49 +572,147 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         dq_raw = *reinterpret_cast<const u32x2 *>(lds + OFF_STG + (m & 1) * STG_BYTES + key * DN + 8 * l);
         dq_sc = *reinterpret_cast<const float *>(lds + OFF_SC + (m & 1) * SC_BYTES + key * 16 + 4 * (l >> 4));
     };
-    auto dequant_write = [&](const int tb, const int kk) {
-        const int key = 8 * w + kk;
-        dequant8((int)dq_raw[0], (int)dq_raw[1], dq_sc, reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb * TILE_BYTES) + key * NPITCH + 8 * l);
+    // The same as a piece of vector work for the 36 slots of the S^T product (see gemm1): slot ks
+    // converts quarter ks % 4 of key ks / 4; dequant_read(m, 0) must have been issued before.
+    u32x2 dqm_raw;
+    float dqm_sc, dqm_bias;
+    u32x4 dqm_out;
+    uint32_t dqm_v = 0;
+    auto dequant_micro = [&](const int ks, const int m, const int tb) {
+        const int g = ks >> 2, e = ks & 3;
+        if (g >= 8) return;
+        if (e == 0) {
+            dqm_raw = dq_raw;
+            dqm_sc = dq_sc;
+            if (g + 1 < 8) dequant_read(m, g + 1);
+            dqm_bias = -128.0f * dqm_sc;
+        }
+        if ((e & 1) == 0) dqm_v = dqm_raw[e >> 1] ^ 0x80808080u;
+        // same arithmetic as dequant8: fma(float(byte + 128), sc, -128*sc) rounds x*sc once
+        const float f0 = __builtin_fmaf((float)((dqm_v >> (16 * (e & 1))) & 0xffu), dqm_sc, dqm_bias);
+        const float f1 = __builtin_fmaf((float)((dqm_v >> (16 * (e & 1) + 8)) & 0xffu), dqm_sc, dqm_bias);
+        dqm_out[e] = pack_bf16x2(f0, f1);
+        if (e == 3)
+            *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb * TILE_BYTES) + (8 * w + g) * NPITCH + 8 * l) = dqm_out;
     };
-    auto dequant_key = [&](const int m, const int tb, const int kk) {
-        dequant_read(m, kk);
-        dequant_write(tb, kk);
+    // a whole tile share at once (pipeline fill): all reads first, then the conversions
+    auto dequant_tile = [&](const int m, const int tb) {
+        u32x2 raw[8];
+        float sc[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const int key = 8 * w + kk;
+            raw[kk] = *reinterpret_cast<const u32x2 *>(lds + OFF_STG + (m & 1) * STG_BYTES + key * DN + 8 * l);
+            sc[kk] = *reinterpret_cast<const float *>(lds + OFF_SC + (m & 1) * SC_BYTES + key * 16 + 4 * (l >> 4));
+        }
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+            dequant8((int)raw[kk][0], (int)raw[kk][1], sc[kk],
+                     reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb * TILE_BYTES) + (8 * w + kk) * NPITCH + 8 * l);
     };
 
-    if (nt > 0) request_tile(0);
-    if (nt > 1) request_tile(1);
-
-    // ---- Q^T fragments: lane (head, half) holds q[head][16*ks + 8*half .. +8], staged per wave (its own
-    // 32 heads) in two passes.  Slot s of a pass is chunk s % 37 of head s / 37 (chunk 36 is padding);
-    // heads past NQ read the last head and are never stored.
+    // ---- prologue.  Everything that does not depend on anything else is requested at once: the first
+    // half of Q^T, the top-k indices of the split and the sequence's block-table row.  Then, as the
+    // data arrives: Q^T half 1 -> registers, Q^T half 2 requested, row table built (LDS lookups),
+    // tiles 0 and 1 requested, Q^T half 2 -> registers.
+    //
+    // Q^T fragments: lane (head, half) holds q[head][16*ks + 8*half .. +8], staged per wave (its own 32
+    // heads) in two passes: nope chunks 0..31 of every head, then nope chunks 32..63 plus the 8 rope
+    // chunks.  A nope request covers two heads (lane = 32*(head & 1) + position), a rope request
+    // eight (lane = 8*(head & 7) + position); position pos of head h holds chunk pos ^ (h & 7), which
+    // makes the fragment reads conflict-free.  The cache address is a wave-uniform base plus a
+    // per-lane offset.  Heads past NQ read the last head and are never stored.
     bf16x8 qf[KSTEPS];
-    {
-        const uint32_t qdst = lds0 + OFF_TILE + w * QREGION;
-        const uint8_t *qsrc = lds + OFF_TILE + w * QREGION + col * QPITCH + 16 * half;
-#pragma unroll
-        for (int pass = 0; pass < 2; ++pass) {
+    const uint32_t qdst = lds0 + OFF_TILE + w * QREGION;
+    const int q_head0 = hg * 128 + w * 32;
+    const bool q_all = q_head0 + 32 <= p.NQ;                          // wave-uniform: all 32 heads exist
+    auto request_q = [&](const int pass) {
+        const size_t qrow0 = (size_t)t * p.NQ + q_head0;
+        if (q_all) {
 #pragma unroll 1
-            for (int i = 0; i < QINSTR; ++i) {
-                const int sl = i * 64 + l;
-                int hl = sl / (QCHUNKS + 1);
-                int c = sl - hl * (QCHUNKS + 1);
-                hl = hl > 31 ? 31 : hl;
-                c = c >= QCHUNKS ? 0 : c;
-                int hd = hg * 128 + w * 32 + hl;
-                hd = hd < p.NQ ? hd : p.NQ - 1;
-                const size_t qrow = (size_t)t * p.NQ + hd;
-                const int dim = pass * (8 * QCHUNKS) + 8 * c;         // first of the chunk's 8 contraction dims
-                const uint16_t *src = dim < DN ? p.q_nope + qrow * DN + dim : p.q_rope + qrow * DR + (dim - DN);
-                dma16(src, qdst + i * 1024);
+            for (int i = 0; i < 16; ++i) {
+                const int h = 2 * i + half;
+                const uint32_t off = (uint32_t)(half * (DN * 2) + (((pass * 32) + (col ^ (h & 7))) << 4));
+                dma16_base(p.q_nope + (qrow0 + 2 * i) * DN, off, qdst + i * 1024);
             }
-            __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0)
-            asm volatile("" ::: "memory");
+            if (pass == 1) {
+                const uint32_t off = (uint32_t)((l >> 3) * (DR * 2) + (((l & 7) ^ (l >> 3)) << 4));
+#pragma unroll 1
+                for (int j = 0; j < 4; ++j) dma16_base(p.q_rope + (qrow0 + 8 * j) * DR, off, qdst + 16 * 1024 + j * 1024);
+            }
+        } else {
+#pragma unroll 1
+            for (int i = 0; i < 16; ++i) {
+                const int h = 2 * i + half;
+                int hd = q_head0 + h;
+                hd = hd < p.NQ ? hd : p.NQ - 1;
+                dma16(p.q_nope + ((size_t)t * p.NQ + hd) * DN + 8 * ((pass * 32) + (col ^ (h & 7))), qdst + i * 1024);
+            }
+            if (pass == 1) {
+#pragma unroll 1
+                for (int j = 0; j < 4; ++j) {
+                    const int h = 8 * j + (l >> 3);
+                    int hd = q_head0 + h;
+                    hd = hd < p.NQ ? hd : p.NQ - 1;
+                    dma16(p.q_rope + ((size_t)t * p.NQ + hd) * DR + 8 * ((l & 7) ^ (l >> 3)), qdst + 16 * 1024 + j * 1024);
+                }
+            }
+        }
+    };
+    auto collect_q = [&](const int pass) {
+        const uint8_t *qn = lds + OFF_TILE + w * QREGION + col * 512;
+        const uint8_t *qr = lds + OFF_TILE + w * QREGION + 16 * 1024 + col * 128;
+        asm volatile("" ::: "memory");
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS / 2; ++ks) qf[pass * (KSTEPS / 2) + ks] = *reinterpret_cast<const bf16x8 *>(qsrc + 32 * ks);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_waitcnt(0xC07F);                       // lgkmcnt(0): the region may be overwritten
+        for (int ks = 0; ks < 16; ++ks) qf[16 * pass + ks] = *reinterpret_cast<const bf16x8 *>(qn + (((2 * ks + half) ^ (col & 7)) << 4));
+        if (pass == 1) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) qf[32 + ks] = *reinterpret_cast<const bf16x8 *>(qr + (((2 * ks + half) ^ (col & 7)) << 4));
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);                           // lgkmcnt(0): the region may be overwritten
+    };
+    request_q(0);
+
+    // top-k indices of the split (at most four per thread) and the block-table row.  Keys past k_end in
+    // the last tile repeat the split's first key (finite data, masked out of the softmax).
+    constexpr int IDX_PER_THREAD = SFA_PIPE_MAX_CHUNK / 256;
+    int idxr[IDX_PER_THREAD];
+#pragma unroll
+    for (int q = 0; q < IDX_PER_THREAD; ++q) {
+        const int i = tid + 256 * q;
+        idxr[q] = i < nt * KT ? p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)] : 0;
+    }
+    int *const bt_lds = reinterpret_cast<int *>(lds + OFF_P);        // the P^T area is idle until the loop
+    const bool bt_cached = p.maxblk <= P_BYTES / 4;
+    if (bt_cached)
+        for (int i = tid; i < p.maxblk; i += 256) bt_lds[i] = p.bt[(size_t)b * p.maxblk + i];
+    // (the compiler waits for these loads before it uses them; requests complete in order, so the first
+    // half of Q^T has landed by then as well)
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < IDX_PER_THREAD; ++q) {
+        const int i = tid + 256 * q;
+        if (i < nt * KT) {
+            const int idx = idxr[q];
+            int blk = idx / p.bs;
+            blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
+            const int phys = bt_cached ? bt_lds[blk] : p.bt[(size_t)b * p.maxblk + blk];
+            long long row = (long long)phys * p.bs + (idx - (idx / p.bs) * p.bs);
+            row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
+            rows_lds[i] = (int)row;
         }
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);                               // vmcnt(0): Q^T half 1 (and all else) landed
+    collect_q(0);
+    request_q(1);
+    __syncthreads();                                                  // row table complete
+    if (nt > 0) request_tile(0);
+    if (nt > 1) request_tile(1);
+    if (nt > 1) __builtin_amdgcn_s_waitcnt(0x0F7C);                   // vmcnt(12): Q^T half 2 landed, tiles may be in flight
+    else if (nt > 0) __builtin_amdgcn_s_waitcnt(0x0F76);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
+    collect_q(1);
     __syncthreads();                                                  // the tile area is free
 
     f32x16 o[DVB];
@@ -718,28 +807,32 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         }
     };
 
-    // ---- pipeline fill: tiles 0 and 1 de-quantised, tiles 2 and 3 requested, S(0) and its softmax
+    // ---- pipeline fill: tile 0 de-quantised, S(0) with the de-quantisation of tile 1 between its
+    // products, tiles 2 and 3 requested as soon as their staging buffers are free, softmax of S(0)
     f32x16 s;
     bf16x8 pf_cur[2], pf_next[2];
     if (nt > 0) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+        if (nt > 1) __builtin_amdgcn_s_waitcnt(0x0F76);               // vmcnt(6): tile 0 staged, tile 1 may be in flight
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
         asm volatile("" ::: "memory");
-#pragma unroll
-        for (int kk = 0; kk < 8; ++kk) dequant_key(0, 0, kk);
-        if (nt > 1) {
-#pragma unroll
-            for (int kk = 0; kk < 8; ++kk) dequant_key(1, 1, kk);
-        }
+        dequant_tile(0, 0);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);
         if (nt > 2) request_tile(2);
-        if (nt > 3) request_tile(3);
         __syncthreads();
-        gemm1(0, 0, s, [](int) {});
+        if (nt > 2) __builtin_amdgcn_s_waitcnt(0x0F76);               // tile 1 staged
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+        dequant_read(1, 0);
+        gemm1(0, 0, s, [&](const int ks) { dequant_micro(ks, 1, 1); });
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        if (nt > 3) request_tile(3);
         mask_tail(k_begin, s);
 #pragma unroll
         for (int m = 0; m < 32; ++m) softmax_micro(m, s, pf_cur);
         sm_rescale = false;
+        __syncthreads();                                              // tile 1 complete
     }
 
     float *const alpha_tab = reinterpret_cast<float *>(lds + OFF_ALPHA);
@@ -766,30 +859,7 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         asm volatile("" ::: "memory");
         dequant_read(n + 2, 0);
-        {
-            u32x2 raw;
-            float sc, bias;
-            u32x4 outv;
-            uint32_t v = 0;
-            gemm1(tb_next, (n + 1) & 3, s, [&](const int ks) {
-                const int g = ks >> 2, e = ks & 3;               // key g of the wave's eight, quarter e of its 8 values
-                if (g >= 8) return;
-                if (e == 0) {
-                    raw = dq_raw;
-                    sc = dq_sc;
-                    if (g + 1 < 8) dequant_read(n + 2, g + 1);
-                    bias = -128.0f * sc;
-                }
-                if ((e & 1) == 0) v = raw[e >> 1] ^ 0x80808080u;
-                // same arithmetic as dequant8: fma(float(byte + 128), sc, -128*sc) rounds x*sc once
-                const float f0 = __builtin_fmaf((float)((v >> (16 * (e & 1))) & 0xffu), sc, bias);
-                const float f1 = __builtin_fmaf((float)((v >> (16 * (e & 1) + 8)) & 0xffu), sc, bias);
-                outv[e] = pack_bf16x2(f0, f1);
-                if (e == 3)
-                    *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(lds + OFF_TILE + tb_fill * TILE_BYTES) +
-                                               (8 * w + g) * NPITCH + 8 * l) = outv;
-            });
-        }
+        gemm1(tb_next, (n + 1) & 3, s, [&](const int ks) { dequant_micro(ks, n + 2, tb_fill); });
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): the staging buffer has been read
         if (n + 4 < nt) request_tile(n + 4);
@@ -843,9 +913,9 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
 
     // ---- epilogue.  Wave w holds value channels 128*w .. +127 of all 128 heads: accumulator
     // o[4*i + hb], lane (head, half) = channels 128*w + 32*i + 8*(r/4) + 4*half + r%4 of head 32*hb + head.
-    // One head block at a time goes through the wave's slice of the (now idle) tile area, 32 heads x
-    // 128 channels fp32 with 16-byte chunk c of head h at chunk c ^ (h & 7), so that 32 lanes write
-    // 256 contiguous bytes of one head.  The 1/l factors of all heads are shared through LDS.
+    // One head block at a time, scaled by 1/l and rounded to the 16-bit output type, goes through the
+    // wave's slice of the (now idle) tile area, so that 32 lanes write 256 contiguous bytes of one
+    // head.  The 1/l factors of all heads are shared through LDS.
     mfma_to_valu_fence();
     {
         float *stage = reinterpret_cast<float *>(lds) + w * (32 * 128);
@@ -865,33 +935,33 @@ __global__ __launch_bounds__(256) void sfa_decode_pipelined_kernel(const SfaPara
             const int head_base = hg * 128 + 32 * HB;
             uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 128 * w + 4 * col
                                    : p.part_o + (prow_base + head_base + half) * DN + 128 * w + 4 * col;
+            const float inv = inv_tab[32 * HB + col];               // this lane's head of the block
+            // staged as 16-bit values: 8-byte chunk c (4 channels) of head h at chunk c ^ (h & 15)
+            uint8_t *st = reinterpret_cast<uint8_t *>(stage);
 #pragma unroll
             for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     const f32x16 &acc = o[4 * b4 + HB];
-                    const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
-                    *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
+                    const float v0 = acc[4 * q4] * inv, v1 = acc[4 * q4 + 1] * inv, v2 = acc[4 * q4 + 2] * inv, v3 = acc[4 * q4 + 3] * inv;
+                    u32x2 pk;
+                    pk[0] = FINAL ? pack_bf16x2(v0, v1) : pack_f16x2(v0, v1);
+                    pk[1] = FINAL ? pack_bf16x2(v2, v3) : pack_f16x2(v2, v3);
+                    *reinterpret_cast<u32x2 *>(st + col * 256 + (((8 * b4 + 2 * q4 + half) ^ (col & 15)) << 3)) = pk;
                 }
 #pragma unroll 1
             for (int pq = 0; pq < 2; ++pq) {
-                f32x4 rv[8];
-                float iv[8];
+                u32x2 rv[8];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int hl = 2 * (8 * pq + e) + half;
-                    rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
-                    iv[e] = inv_tab[32 * HB + hl];
+                    rv[e] = *reinterpret_cast<const u32x2 *>(st + hl * 256 + ((col ^ (hl & 15)) << 3));
                 }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int hl = 2 * (8 * pq + e) + half;
-                    const f32x4 v = rv[e] * iv[e];
-                    u32x2 pk;
-                    pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
-                    pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
                     if (ALL || head_base + hl < p.NQ)
-                        *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN) = pk;
+                        *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN) = rv[e];
                 }
             }
         };
