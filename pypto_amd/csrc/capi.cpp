@@ -71,8 +71,7 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
     pl.hgroups = (int)((a->nq + heads_per_wg - 1) / heads_per_wg);
     const long long rows = a->b * a->s1;
     const int tiles = (int)((a->topk + pto::SFA_KEY_TILE - 1) / pto::SFA_KEY_TILE);
-    const int max_chunk = pl.waves == 4 ? pto::SFA_PIPE_MAX_CHUNK : pto::SFA_MAX_CHUNK;
-    const int min_split = (int)((a->topk + max_chunk - 1) / max_chunk);
+    const int min_split = (int)((a->topk + pto::SFA_MAX_CHUNK - 1) / pto::SFA_MAX_CHUNK);
     int ns = a->num_splits;
     if (ns == 0) {
         // fill the chip once; a split shorter than four tiles is all prologue

@@ -6,7 +6,6 @@
 namespace pto {
 
 constexpr int SFA_MAX_CHUNK = 2048;   // most keys one workgroup handles (row-translation table in LDS)
-constexpr int SFA_PIPE_MAX_CHUNK = 1024;   // the same for the pipelined kernel (workgroups of 128 heads)
 constexpr int SFA_KEY_TILE = 32;
 
 struct SfaParams {
