@@ -492,7 +492,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 }
 
 // Merges the key splits of one query row: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - m)
-// and O_s the split's normalised fp16 partial.  One thread per (row, head, 8 value channels).
+// and O_s the split's normalised fp16 partial (all zeros for an empty split, whose weight is zero).
+// One thread per (row, head, 8 value channels); splits are taken eight at a time with all their loads
+// in flight together.
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
 {
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -502,29 +504,43 @@ __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
     const size_t th = gid / (DN / 8);
     const int head = (int)(th % p.NQ);
     const int t = (int)(th / p.NQ);
+    const size_t prow0 = (size_t)t * p.nsplit * p.NQ + head;       // split s: prow0 + s * NQ
+    const f32x2 *ml = reinterpret_cast<const f32x2 *>(p.part_ml);
+
     float m = -INFINITY;
-    for (int s = 0; s < p.nsplit; ++s) {
-        const size_t prow = ((size_t)t * p.nsplit + s) * p.NQ + head;
-        if (p.part_ml[prow * 2 + 1] > 0.f) m = fmaxf(m, p.part_ml[prow * 2]);
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        f32x2 v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = ml[prow0 + (size_t)(s0 + e < p.nsplit ? s0 + e : p.nsplit - 1) * p.NQ];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (v[e][1] > 0.f) m = fmaxf(m, v[e][0]);
     }
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float wsum = 0.f;
-    for (int s = 0; s < p.nsplit; ++s) {
-        const size_t prow = ((size_t)t * p.nsplit + s) * p.NQ + head;
-        const float ls = p.part_ml[prow * 2 + 1];
-        if (ls > 0.f) {
-            const float wgt = ls * __builtin_amdgcn_exp2f(p.part_ml[prow * 2] - m);
-            const f16x8 hv = *reinterpret_cast<const f16x8 *>(p.part_o + prow * DN + 8 * c8);
+    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
+        f32x2 v[8];
+        f16x8 hv[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[e] += wgt * (float)hv[e];
+        for (int e = 0; e < 8; ++e) {
+            const size_t prow = prow0 + (size_t)(s0 + e < p.nsplit ? s0 + e : p.nsplit - 1) * p.NQ;
+            v[e] = ml[prow];
+            hv[e] = *reinterpret_cast<const f16x8 *>(p.part_o + prow * DN + 8 * c8);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const bool live = s0 + e < p.nsplit && v[e][1] > 0.f;
+            const float wgt = live ? v[e][1] * __builtin_amdgcn_exp2f(v[e][0] - m) : 0.f;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[c] += wgt * (float)hv[e][c];
             wsum += wgt;
         }
     }
     const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
-    u32x4 v;
+    u32x4 outv;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = pack_bf16x2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
-    *reinterpret_cast<u32x4 *>(p.out + ((size_t)t * p.NQ + head) * DN + 8 * c8) = v;
+    for (int e = 0; e < 4; ++e) outv[e] = pack_bf16x2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+    *reinterpret_cast<u32x4 *>(p.out + ((size_t)t * p.NQ + head) * DN + 8 * c8) = outv;
 }
 
 }  // namespace
