@@ -11,6 +11,7 @@ timed region.  Prints ONE JSON line:
                  / average launch duration from HIP events on the launch stream, against 2.5 PFLOP/s;
                  the HBM-side figure (algorithmic bytes / same duration, against 8 TB/s) is in
                  "roofline_hbm" because the shape sits at the ridge of the two
+  packed_cache   the same step through sparse_attention_antiquant_d (one 656-byte row per key)
   indexer        time of one lightning-indexer pass (score + select) on the same batch and on the
                  indexer-only configuration (B=4, KV 32768), with its HBM fraction
   cpu_baseline   the scalar C statement of the golden, all host threads, on a bounded sample of the
@@ -168,6 +169,22 @@ def main():
     achieved_tflops = flops / (ev_avg_ms * 1e-3) / 1e12
     achieved_gbs = byt / (ev_avg_ms * 1e-3) / 1e9
 
+    # ------------------------------------------------------------------ the same step over packed cache rows
+    from pypto_amd.synthetic import pack_nope_cache
+    packed = pack_nope_cache(sfa_d.key_nope_2d, sfa_d.key_rope_2d, sfa_d.k_nope_scales)
+    out_p = torch.zeros_like(out)
+
+    def packed_step(i):
+        pypto_amd.sparse_attention_antiquant_d(sfa_d.query_nope, sfa_d.query_rope, packed, sel[i % ROT],
+                                               sfa_d.block_table, sfa_d.kv_act_seqs, out_p, NQ, 1,
+                                               sfa.softmax_scale, K, 128, sfa.max_blocknum_perbatch, None)
+    _, packed_avg_ms, _ = time_events(packed_step, max(args.steps // 2, 5), 5, torch)
+    sfa_step(0)
+    packed_step(0)
+    torch.cuda.synchronize()
+    packed_same = bool(torch.equal(out.view(torch.int16), out_p.view(torch.int16)))
+    del packed
+
     # ------------------------------------------------------------------ indexer timings
     res = torch.empty([B, 1, K], dtype=torch.int32, device=dev)
 
@@ -230,6 +247,8 @@ def main():
                      "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "flops_per_launch": flops},
         "roofline_hbm": {"bound": "hbm", "achieved": achieved_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": achieved_gbs / PEAK_HBM_GBS, "bytes_per_launch": byt},
+        "packed_cache": {"operator": "sparse_attention_antiquant_d", "us_per_step": packed_avg_ms * 1e3,
+                         "bit_identical_to_three_array_result": packed_same},
         "indexer": {"configs[2]_us_per_step": li2_avg_ms * 1e3, "configs[2]_hbm_frac": li2_bytes / (li2_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     "configs[1]_us_per_step": li1_avg_ms * 1e3, "configs[1]_hbm_frac": li1_bytes / (li1_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes, "scale_dtype": "fp32", "weight_dtype": "bf16"},

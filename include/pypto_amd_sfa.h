@@ -21,6 +21,11 @@
  *       499-538), i.e. what python/pypto/runtime.py:153 dispatches through
  *       ExportedOperatorDeviceLaunchOnceWithDeviceTensorData
  *       (framework/src/machine/runtime/device_launcher_binding.h:204-209).
+ *   pto_sa_antiquant_launch
+ *       the device execution of sparse_attention_antiquant_d / _p
+ *       (examples/models/deepseek_v32_exp/sparse_attention_antiquant_impl.py:263-300,
+ *       322-359), same dispatch point: the same attention over the packed cache
+ *       layout (one 656-byte row per key).
  *   pto_li_decode_launch
  *       the device execution of lightning_indexer_decode
  *       (examples/models/deepseek_v32_exp/lightning_indexer_quant_impl.py:315-346),
@@ -100,6 +105,43 @@ typedef struct PtoSfaQuantArgs {
 
 int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *args, size_t *bytes);
 int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
+
+/*
+ * The same attention over the packed cache of sparse_attention_antiquant_d
+ * (sparse_attention_antiquant_impl.py:45-85 in the reference example; packing
+ * deepseekv32_sparse_attention_antiquant.py:258-268):
+ *
+ *   nope_cache [kv_rows, 656] int8: bytes 0..511 the int8 latent values,
+ *                                   512..639 the 64 bf16 rope values,
+ *                                   640..655 the 4 fp32 scales
+ *
+ * All other tensors, the arithmetic, cur_seq, clamping, constraints, workspace
+ * and num_splits are those of PtoSfaQuantArgs.
+ */
+typedef struct PtoSaAntiquantArgs {
+    const void *query_nope;
+    const void *query_rope;
+    const void *nope_cache;
+    const int32_t *topk_indices;
+    const int32_t *block_table;
+    const int32_t *kv_act_seqs;
+    void *attention_out;
+    void *workspace;
+    size_t workspace_bytes;
+    int64_t b;
+    int64_t s1;
+    int64_t nq;
+    int64_t n_kv;
+    int64_t topk;
+    int64_t block_size;
+    int64_t max_blocknum_perbatch;
+    int64_t kv_rows;
+    float softmax_scale;
+    int32_t num_splits;
+} PtoSaAntiquantArgs;
+
+int pto_sa_antiquant_workspace_bytes(const PtoSaAntiquantArgs *args, size_t *bytes);
+int pto_sa_antiquant_launch(const PtoSaAntiquantArgs *args, void *hip_stream);
 
 /*
  * Lightning indexer, decode form (lightning_indexer_quant_impl.py:52-82 in the

@@ -205,3 +205,24 @@ def sfa_literal_loops(q, kn, kr, kn_scales, topk_indices, block_table, actual_se
             o = torch.matmul((p / l).to(dtype).to(torch.float32), kn_t.to(torch.float32))
             out[b_idx, s1_idx] = o.to(dtype)
     return out
+
+
+def unpack_nope_cache(nope_cache_2d: torch.Tensor):
+    """``[rows, 656] int8`` -> (kn [rows,512] int8, kr [rows,64] bf16, scales [rows,4] fp32): the byte
+    ranges the packed-cache golden reads (deepseekv32_sparse_attention_antiquant.py:109-118:
+    ``[:, :512]`` int8, ``[:, 512:640]`` viewed as the activation dtype, ``[:, 640:]`` viewed as fp32)."""
+    rows = nope_cache_2d.shape[0]
+    kn = nope_cache_2d[:, :512].contiguous()
+    kr = nope_cache_2d[:, 512:640].contiguous().view(torch.bfloat16).reshape(rows, 64)
+    sc = nope_cache_2d[:, 640:656].contiguous().view(torch.float32).reshape(rows, 4)
+    return kn, kr, sc
+
+
+def sa_antiquant_single_pass(q, nope_cache_2d, topk_indices, block_table, actual_seq: Sequence[int],
+                             block_size: int, scalar: float, topk: int) -> torch.Tensor:
+    """Golden of the packed-cache operator, compute_attention_aq
+    (deepseekv32_sparse_attention_antiquant.py:49-136): gather whole 656-byte rows, split them, then
+    exactly the arithmetic of the three-array golden (dequant :109-118, scores :121, softmax :124-130,
+    PV :133).  The reference runs it with s2_tile == topk (:283), where its tile loop is one pass."""
+    kn, kr, sc = unpack_nope_cache(nope_cache_2d)
+    return sfa_single_pass(q, kn, kr, sc, topk_indices, block_table, actual_seq, block_size, scalar, topk)

@@ -3,6 +3,7 @@
 Operators (same names and signatures as the reference examples they replace):
 
 * :func:`sparse_flash_attention_quant_d` / :func:`sparse_flash_attention_quant_p`
+* :func:`sparse_attention_antiquant_d` / :func:`sparse_attention_antiquant_p` (packed 656-byte cache rows)
 * :func:`lightning_indexer_decode`
 
 plus :func:`from_torch`, the tensor hand-over of the reference's jit convention.  The computation
@@ -11,6 +12,7 @@ fallback.
 """
 from .converter import Tensor, from_torch  # noqa: F401
 from .lightning_indexer_quant_impl import LightningIndexerConfigs, lightning_indexer_decode  # noqa: F401
+from .sparse_attention_antiquant_impl import sparse_attention_antiquant_d, sparse_attention_antiquant_p  # noqa: F401
 from .sparse_flash_attention_quant_impl import (SaTileShapeConfig, sparse_flash_attention_quant_d,  # noqa: F401
                                                 sparse_flash_attention_quant_p)
 

@@ -93,6 +93,77 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
     return pl;
 }
 
+constexpr int PACKED_ROW_BYTES = 656;     // 512 int8 | 64 bf16 | 4 fp32
+
+// the packed-cache arguments seen as the three-array ones (the cache pointers are filled in by the caller)
+PtoSfaQuantArgs unpacked_view(const PtoSaAntiquantArgs *a)
+{
+    PtoSfaQuantArgs q;
+    std::memset(&q, 0, sizeof(q));
+    q.query_nope = a->query_nope;
+    q.query_rope = a->query_rope;
+    q.key_nope_2d = a->nope_cache;
+    q.key_rope_2d = a->nope_cache;
+    q.k_nope_scales = a->nope_cache;
+    q.topk_indices = a->topk_indices;
+    q.block_table = a->block_table;
+    q.kv_act_seqs = a->kv_act_seqs;
+    q.attention_out = a->attention_out;
+    q.workspace = a->workspace;
+    q.workspace_bytes = a->workspace_bytes;
+    q.b = a->b;
+    q.s1 = a->s1;
+    q.nq = a->nq;
+    q.n_kv = a->n_kv;
+    q.topk = a->topk;
+    q.block_size = a->block_size;
+    q.max_blocknum_perbatch = a->max_blocknum_perbatch;
+    q.kv_rows = a->kv_rows;
+    q.softmax_scale = a->softmax_scale;
+    q.num_splits = a->num_splits;
+    return q;
+}
+
+// checked arguments -> kernel parameters -> launch; the cache is given as three (base, row pitch) pairs
+int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const uint8_t *kr, int kr_pitch, const uint8_t *ksc,
+                int ksc_pitch, void *hip_stream)
+{
+    const SfaPlan pl = sfa_plan(a);
+    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
+    if (need > 0 && (!a->workspace || a->workspace_bytes < need))
+        return fail(PTO_E_WORKSPACE, "sfa: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+
+    pto::SfaParams p;
+    p.q_nope = static_cast<const uint16_t *>(a->query_nope);
+    p.q_rope = static_cast<const uint16_t *>(a->query_rope);
+    p.kn = kn;
+    p.kr = kr;
+    p.ksc = ksc;
+    p.kn_pitch = kn_pitch;
+    p.kr_pitch = kr_pitch;
+    p.ksc_pitch = ksc_pitch;
+    p.topk_idx = a->topk_indices;
+    p.bt = a->block_table;
+    p.act = a->kv_act_seqs;
+    p.out = static_cast<uint16_t *>(a->attention_out);
+    p.part_o = static_cast<uint16_t *>(a->workspace);
+    p.part_ml = need > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
+    p.kv_rows = a->kv_rows;
+    p.T = (int)(a->b * a->s1);
+    p.S1 = (int)a->s1;
+    p.NQ = (int)a->nq;
+    p.topk = (int)a->topk;
+    p.bs = (int)a->block_size;
+    p.maxblk = (int)a->max_blocknum_perbatch;
+    p.nsplit = pl.nsplit;
+    p.hgroups = pl.hgroups;
+    p.waves = pl.waves;
+    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    hipError_t e = pto::sfa_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "sfa: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
 int li_check(const PtoLiDecodeArgs *a)
 {
     if (!a) return fail(PTO_E_INVALID_ARG, "li: args is NULL");
@@ -145,37 +216,29 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *a, void *hip_stream)
     if (!a->query_nope || !a->query_rope || !a->key_nope_2d || !a->key_rope_2d || !a->k_nope_scales || !a->topk_indices ||
         !a->block_table || !a->kv_act_seqs || !a->attention_out)
         return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
-    const SfaPlan pl = sfa_plan(a);
-    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
-    if (need > 0 && (!a->workspace || a->workspace_bytes < need))
-        return fail(PTO_E_WORKSPACE, "sfa: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+    return sfa_enqueue(a, static_cast<const int8_t *>(a->key_nope_2d), 512, static_cast<const uint8_t *>(a->key_rope_2d), 128,
+                       static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream);
+}
 
-    pto::SfaParams p;
-    p.q_nope = static_cast<const uint16_t *>(a->query_nope);
-    p.q_rope = static_cast<const uint16_t *>(a->query_rope);
-    p.kn = static_cast<const int8_t *>(a->key_nope_2d);
-    p.kr = static_cast<const uint16_t *>(a->key_rope_2d);
-    p.ksc = static_cast<const float *>(a->k_nope_scales);
-    p.topk_idx = a->topk_indices;
-    p.bt = a->block_table;
-    p.act = a->kv_act_seqs;
-    p.out = static_cast<uint16_t *>(a->attention_out);
-    p.part_o = static_cast<uint16_t *>(a->workspace);
-    p.part_ml = need > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
-    p.kv_rows = a->kv_rows;
-    p.T = (int)(a->b * a->s1);
-    p.S1 = (int)a->s1;
-    p.NQ = (int)a->nq;
-    p.topk = (int)a->topk;
-    p.bs = (int)a->block_size;
-    p.maxblk = (int)a->max_blocknum_perbatch;
-    p.nsplit = pl.nsplit;
-    p.hgroups = pl.hgroups;
-    p.waves = pl.waves;
-    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
-    hipError_t e = pto::sfa_launch(p, static_cast<hipStream_t>(hip_stream));
-    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "sfa: launch failed: %s", hipGetErrorString(e));
-    return PTO_OK;
+int pto_sa_antiquant_workspace_bytes(const PtoSaAntiquantArgs *a, size_t *bytes)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "sfa: args is NULL");
+    const PtoSfaQuantArgs q = unpacked_view(a);
+    return pto_sfa_quant_workspace_bytes(&q, bytes);
+}
+
+int pto_sa_antiquant_launch(const PtoSaAntiquantArgs *a, void *hip_stream)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "sfa: args is NULL");
+    const PtoSfaQuantArgs q = unpacked_view(a);
+    int rc = sfa_check(&q);
+    if (rc != PTO_OK) return rc;
+    if (!a->query_nope || !a->query_rope || !a->nope_cache || !a->topk_indices || !a->block_table || !a->kv_act_seqs ||
+        !a->attention_out)
+        return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
+    const uint8_t *base = static_cast<const uint8_t *>(a->nope_cache);
+    return sfa_enqueue(&q, reinterpret_cast<const int8_t *>(base), PACKED_ROW_BYTES, base + 512, PACKED_ROW_BYTES, base + 640,
+                       PACKED_ROW_BYTES, hip_stream);
 }
 
 int pto_li_decode_workspace_bytes(const PtoLiDecodeArgs *a, size_t *bytes)

@@ -120,6 +120,34 @@ PYBIND11_MODULE(_C, m)
               check(pto_sfa_quant_launch(&a, ptr<void>(stream)));
           });
 
+    m.def("sa_antiquant_launch",
+          [](std::uintptr_t query_nope, std::uintptr_t query_rope, std::uintptr_t nope_cache, std::uintptr_t topk_indices,
+             std::uintptr_t block_table, std::uintptr_t kv_act_seqs, std::uintptr_t attention_out, std::uintptr_t workspace,
+             size_t workspace_bytes, int64_t b, int64_t s1, int64_t nq, int64_t n_kv, int64_t topk, int64_t block_size,
+             int64_t max_blocknum_perbatch, int64_t kv_rows, double softmax_scale, int num_splits, std::uintptr_t stream) {
+              PtoSaAntiquantArgs a{};
+              a.query_nope = ptr<const void>(query_nope);
+              a.query_rope = ptr<const void>(query_rope);
+              a.nope_cache = ptr<const void>(nope_cache);
+              a.topk_indices = ptr<const int32_t>(topk_indices);
+              a.block_table = ptr<const int32_t>(block_table);
+              a.kv_act_seqs = ptr<const int32_t>(kv_act_seqs);
+              a.attention_out = ptr<void>(attention_out);
+              a.workspace = ptr<void>(workspace);
+              a.workspace_bytes = workspace_bytes;
+              a.b = b;
+              a.s1 = s1;
+              a.nq = nq;
+              a.n_kv = n_kv;
+              a.topk = topk;
+              a.block_size = block_size;
+              a.max_blocknum_perbatch = max_blocknum_perbatch;
+              a.kv_rows = kv_rows;
+              a.softmax_scale = static_cast<float>(softmax_scale);
+              a.num_splits = num_splits;
+              check(pto_sa_antiquant_launch(&a, ptr<void>(stream)));
+          });
+
     m.def("li_decode_workspace_bytes",
           [](int64_t t, int64_t b, int64_t n_heads, int64_t head_dim, int64_t block_num, int64_t block_size,
              int64_t max_blocknum_perbatch, int64_t selected_count, int q_dt, int k_dt, int w_dt) {

@@ -11,9 +11,12 @@ constexpr int SFA_KEY_TILE = 32;
 struct SfaParams {
     const uint16_t *q_nope;   // [T*NQ, 512] bf16
     const uint16_t *q_rope;   // [T*NQ, 64]  bf16
-    const int8_t *kn;         // [kv_rows, 512]
-    const uint16_t *kr;       // [kv_rows, 64] bf16
-    const float *ksc;         // [kv_rows, 4]
+    // The three parts of a cache row, each with its own base and row pitch in bytes: separate arrays
+    // (pitches 512 / 128 / 16) or one packed array of 656-byte rows (512 int8 | 64 bf16 | 4 fp32).
+    const int8_t *kn;         // 512 int8 latent values
+    const uint8_t *kr;        // 64 bf16 rope values
+    const uint8_t *ksc;       // 4 fp32 scales, one per 128 latent channels
+    int kn_pitch, kr_pitch, ksc_pitch;
     const int32_t *topk_idx;  // [T, topk]
     const int32_t *bt;        // [B, maxblk]
     const int32_t *act;       // [B]

@@ -18,7 +18,8 @@
 // (the accumulator layout of a 32x32 product gives lane (head, half) the keys 8*(r/4)+4*half+r%4;
 // the transposed V read uses the same key order, so no cross-lane movement is needed).
 // All NW waves gather and de-quantise the tile cooperatively: each selected row is read once per
-// workgroup (512 B int8 + 128 B rope + 16 B scales) and written to LDS as 576 bf16.
+// workgroup (512 B int8 + 128 B rope + 16 B scales, from three arrays or from one packed 656-byte row)
+// and written to LDS as 576 bf16.
 #include <type_traits>
 
 #include "common.h"
@@ -262,14 +263,14 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 #pragma unroll
         for (int i = 0; i < NP; ++i) {
             const int row = rtab[i];
-            raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * DN + 16 * col);
-            rsc[i] = p.ksc[(size_t)row * 4 + (col >> 3)];
+            raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * p.kn_pitch + 16 * col);
+            rsc[i] = *reinterpret_cast<const float *>(p.ksc + (size_t)row * p.ksc_pitch + 4 * (col >> 3));
         }
 #pragma unroll
         for (int i = 0; i < RP; ++i) {
             const int e = tid + i * NW * 64;
             const int row = rows_lds[(kt - k_begin) + (e >> 3)];
-            rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * DR + 8 * (e & 7));
+            rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * p.kr_pitch + 16 * (e & 7));
         }
     };
     // de-quantise and store one eighth of the gathered tile (piece 0 also stores the rope part)

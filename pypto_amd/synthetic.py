@@ -112,6 +112,18 @@ class SfaInputs:
         return SfaInputs(**kw)
 
 
+def pack_nope_cache(key_nope_2d: torch.Tensor, key_rope_2d: torch.Tensor, k_nope_scales: torch.Tensor) -> torch.Tensor:
+    """The packed cache of the antiquant operator: ``[rows, 656] int8`` = 512 int8 latent values |
+    the 64 bf16 rope values as bytes | the 4 fp32 scales as bytes (the packing of the reference
+    driver, deepseekv32_sparse_attention_antiquant.py:258-268)."""
+    rows = key_nope_2d.shape[0]
+    out = torch.zeros([rows, 656], dtype=torch.int8, device=key_nope_2d.device)
+    out[:, :512] = key_nope_2d
+    out[:, 512:640] = key_rope_2d.contiguous().view(torch.int8).reshape(rows, 128)
+    out[:, 640:] = k_nope_scales.contiguous().view(torch.int8).reshape(rows, 16)
+    return out
+
+
 def gen_sfa_inputs(b: int, s1: int, n_q: int, actual_seq: Sequence[int], topk: int = 2048, seed: int = 0,
                    block_size: int = BLOCK_SIZE, shuffle_table: bool = True,
                    topk_indices: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,

@@ -137,3 +137,40 @@ def test_identical_keys_invariant_full_width():
         v = so.dequant_kn(inp.key_nope_2d[phys:phys + 1], inp.k_nope_scales[phys:phys + 1]).float()
         # softmax over identical scores is uniform; P = bf16(1) and the row sum 2048 are exact
         assert torch.equal(out[bi, 0].float(), v.expand(128, -1))
+
+
+# ------------------------------------------------------------------ packed 656-byte cache rows
+
+def run_packed(inp, entry="d"):
+    from pypto_amd.synthetic import pack_nope_cache
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    packed = pack_nope_cache(d.key_nope_2d, d.key_rope_2d, d.k_nope_scales)
+    out = torch.full([inp.b, inp.s1, inp.n_q, 512], float("nan"), dtype=torch.bfloat16, device=dev)
+    fn = pypto_amd.sparse_attention_antiquant_d if entry == "d" else pypto_amd.sparse_attention_antiquant_p
+    cfg = pypto_amd.SaTileShapeConfig(128, 2048, [128] * 6, [8, 2048], [128] * 6, [64, 128])
+    ret = fn(pypto_amd.from_torch(d.query_nope), pypto_amd.from_torch(d.query_rope), pypto_amd.from_torch(packed),
+             pypto_amd.from_torch(d.topk_indices), pypto_amd.from_torch(d.block_table), pypto_amd.from_torch(d.kv_act_seqs),
+             pypto_amd.from_torch(out, name="out"), inp.n_q, 1, inp.softmax_scale, inp.topk, inp.block_size,
+             inp.max_blocknum_perbatch, cfg)
+    assert ret is None
+    torch.cuda.synchronize()
+    return out.cpu(), packed.cpu()
+
+
+@pytest.mark.parametrize("n_q,b,s1,act,topk,entry", [
+    (128, 2, 1, [5000, 3000], 2048, "d"),      # decode, key splits
+    (16, 1, 1, [4096], 256, "d"),              # the tiny configuration
+    (128, 1, 3, [700], 512, "p"),              # prefill entry, causal rows
+    (40, 3, 2, [300, 1, 64], 128, "d"),        # head count that fills no wave, rows without keys
+])
+def test_packed_cache_operator(n_q, b, s1, act, topk, entry):
+    """sparse_attention_antiquant over packed rows: against its golden, and bit-identical to the
+    three-array operator on the same data (same kernel, other row pitches)."""
+    from oracle import sfa_oracle as so
+    inp = gen_sfa_inputs(b, s1, n_q, act, topk=topk, seed=17 + n_q)
+    out, packed = run_packed(inp, entry)
+    ref = so.sa_antiquant_single_pass(inp.q_bsnd(), packed, inp.topk_indices, inp.block_table, inp.actual_seq,
+                                      inp.block_size, inp.softmax_scale, inp.topk)
+    check(out, ref, f"packed nq={n_q} b={b} s1={s1} act={act} topk={topk}")
+    assert torch.equal(out.view(torch.int16), run_op(inp, entry=entry).view(torch.int16))

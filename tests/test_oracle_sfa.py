@@ -204,3 +204,43 @@ def test_c_statement_agrees_with_torch_statement(c_oracle, tile):
     assert float((d > ulp).float().mean()) == 0.0
     assert float((d > 0).float().mean()) < 0.02
     assert torch.all(got[2, 0] == 0)
+
+
+# ------------------------------------------------------------------ packed 656-byte cache rows
+
+def test_packed_row_byte_layout_known_answer():
+    """A row written byte by byte with struct: 512 int8 | 64 bf16 (little endian) | 4 fp32 (little endian),
+    the layout of the reference driver (deepseekv32_sparse_attention_antiquant.py:258-268)."""
+    import struct
+    from oracle import sfa_oracle as so
+    ints = [((7 * i) % 256) - 128 for i in range(512)]
+    bf16_bits = [0x3F80, 0xC000, 0x0000, 0x8000, 0x7F7F, 0x0001] + [0x3C00 + i for i in range(58)]   # 1.0, -2.0, +0, -0, max, tiny ...
+    scales = [0.0078125, 1e-8, 3.5, 127.0]
+    row = struct.pack("<512b", *ints) + struct.pack("<64H", *bf16_bits) + struct.pack("<4f", *scales)
+    assert len(row) == 656
+    cache = torch.frombuffer(bytearray(row + bytes(656)), dtype=torch.int8).reshape(2, 656)
+    kn, kr, sc = so.unpack_nope_cache(cache)
+    assert kn.dtype == torch.int8 and kn[0].tolist() == ints
+    assert kr.dtype == torch.bfloat16 and kr[0].view(torch.int16).tolist() == [b - 65536 if b >= 32768 else b for b in bf16_bits]
+    assert float(kr[0, 0]) == 1.0 and float(kr[0, 1]) == -2.0
+    assert sc.dtype == torch.float32 and sc[0].tolist() == [struct.unpack("<f", struct.pack("<f", x))[0] for x in scales]
+    assert kn[1].abs().sum() == 0 and sc[1].abs().sum() == 0
+
+
+def test_packed_cache_round_trip_and_golden_equivalence():
+    """pack (generator side) then unpack (oracle side) is the identity, and the packed golden equals the
+    three-array golden on the same data."""
+    from oracle import sfa_oracle as so
+    from pypto_amd.synthetic import gen_sfa_inputs, pack_nope_cache
+    inp = gen_sfa_inputs(2, 2, 8, [300, 70], topk=64, seed=5)
+    packed = pack_nope_cache(inp.key_nope_2d, inp.key_rope_2d, inp.k_nope_scales)
+    assert packed.shape == (inp.key_nope_2d.shape[0], 656) and packed.dtype == torch.int8
+    kn, kr, sc = so.unpack_nope_cache(packed)
+    assert torch.equal(kn, inp.key_nope_2d)
+    assert torch.equal(kr.view(torch.int16), inp.key_rope_2d.view(torch.int16))
+    assert torch.equal(sc.view(torch.int32), inp.k_nope_scales.view(torch.int32))
+    a = so.sa_antiquant_single_pass(inp.q_bsnd(), packed, inp.topk_indices, inp.block_table, inp.actual_seq,
+                                    inp.block_size, inp.softmax_scale, inp.topk)
+    b = so.sfa_single_pass(inp.q_bsnd(), inp.key_nope_2d, inp.key_rope_2d, inp.k_nope_scales, inp.topk_indices,
+                           inp.block_table, inp.actual_seq, inp.block_size, inp.softmax_scale, inp.topk)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
