@@ -287,6 +287,13 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
         const long long pairs = (long long)a->t * ((p.score_stride + 63) / 64);
         long long ppw = pairs / ((long long)cu_count() * 4 * 4);
         p.ppw = (int)(ppw < 1 ? 1 : (ppw > pto::LI_MAX_PAIRS_PER_WAVE ? pto::LI_MAX_PAIRS_PER_WAVE : ppw));
+        // With few query tokens the kernel balances the runs itself from the actual lengths: one round
+        // of resident waves (two workgroups per CU), more only if the longest possible input needs it.
+        p.balanced = a->t <= pto::LI_MAX_BALANCED_TOKENS;
+        long long waves = (long long)cu_count() * 8;
+        const long long need = (pairs + pto::LI_MAX_PAIRS_PER_WAVE - 1) / pto::LI_MAX_PAIRS_PER_WAVE + 2 * a->t;
+        waves = waves > need ? waves : need;
+        p.score_wgs = (int)((waves + 3) / 4);
     }
     hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));

@@ -9,6 +9,7 @@ constexpr int LI_MAX_SELECT = 2048;     // most indices one query token can rece
 constexpr int LI_MAX_SEQ = 128 * 1024;  // longest key sequence
 constexpr int LI_HEADS = 64;
 constexpr int LI_DIM = 128;
+constexpr int LI_MAX_BALANCED_TOKENS = 512; // most query tokens the balanced run mapping of the score kernel handles
 constexpr int LI_MAX_PAIRS_PER_WAVE = 32;  // a wave keeps one cache-row index per 32-key block of its run in a lane
 
 struct LiParams {
@@ -25,6 +26,8 @@ struct LiParams {
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes
     int ppw;                // 64-key block pairs per wave of the score kernel, <= LI_MAX_PAIRS_PER_WAVE
+    int balanced;           // score kernel sizes its runs from the sequence lengths (T <= LI_MAX_BALANCED_TOKENS)
+    int score_wgs;          // its launch size in workgroups of four waves when balanced
 };
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream);

@@ -66,6 +66,58 @@ __device__ __forceinline__ uint32_t score_key(const float x)
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// Wave-wide scan and reductions on DPP (no LDS traffic).  row_shr:n moves a value n lanes up inside
+// its row of 16, row_bcast15/31 carry the last lane of a row / of the lower half-wave upward; lanes
+// without a source keep the identity passed as the old value.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_u32(const uint32_t identity, const uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)identity, (int)v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// inclusive prefix sum over the 64 lanes
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v)
+{
+    v += dpp_u32<0x111, 0xf>(0u, v);
+    v += dpp_u32<0x112, 0xf>(0u, v);
+    v += dpp_u32<0x114, 0xf>(0u, v);
+    v += dpp_u32<0x118, 0xf>(0u, v);
+    v += dpp_u32<0x142, 0xa>(0u, v);
+    v += dpp_u32<0x143, 0xc>(0u, v);
+    return v;
+}
+
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_reduce_bits(uint32_t v, const uint32_t identity, Op op)
+{
+    v = op(v, dpp_u32<0x111, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x112, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x114, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x118, 0xf>(identity, v));
+    v = op(v, dpp_u32<0x142, 0xa>(identity, v));
+    v = op(v, dpp_u32<0x143, 0xc>(identity, v));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);     // lane 63 holds the reduction of all lanes
+}
+
+__device__ __forceinline__ float wave_min(const float x)
+{
+    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0x7f800000u, [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fminf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
+__device__ __forceinline__ float wave_max(const float x)
+{
+    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0xff800000u, [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
+__device__ __forceinline__ uint32_t wave_max_u32(const uint32_t x)
+{
+    return wave_reduce_bits(x, 0u, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+}
+
 // fp32 product of one half of a packed fp16 pair with a wave-uniform fp32 factor, rounded once:
 // v_fma_mix_f32 widens the fp16 operand on the fly.  The addend +0 turns a product of -0 into +0, which
 // no later step can tell apart: the running sum starts at +0 and so never is -0 itself.
@@ -121,19 +173,60 @@ template <int KDT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void li_score_kernel(const LiParams p)
 {
     __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_BUF_BYTES];
-    const int t = blockIdx.y;
-    const int b = t / p.S1;
-    int cur = p.act[b];
-    const int cap = p.maxblk * p.bs;
-    cur = cur < 0 ? 0 : (cur > cap ? cap : cur);
     const int w = threadIdx.x >> 6;
     const int l = threadIdx.x & 63;
     const int j = l & 31;
     const int half = l >> 5;
-    const int key0 = (blockIdx.x * 4 + w) * (p.ppw * 64);
+    const int cap = p.maxblk * p.bs;
+    int t, key0, ppw;
+    if (p.balanced) {
+        // Balanced mapping (at most 512 query tokens): the launch has a fixed number of waves; every wave
+        // reads all sequence lengths, sizes the runs so that the runs of all tokens just fill the
+        // launch, and takes the gw-th run in token order.  Short and long sequences then cost the same
+        // number of trips per wave and the whole pass is one round of resident waves.
+        const int gw = blockIdx.x * 4 + w;
+        const int nwaves = gridDim.x * 4;
+        int pairs[8], total = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int tt = l + 64 * i;
+            int c = tt < p.T ? p.act[tt / p.S1] : 0;
+            c = c < 0 ? 0 : (c > cap ? cap : c);
+            pairs[i] = (c + 63) >> 6;
+            total += pairs[i];
+        }
+        total = (int)wave_incl_scan((uint32_t)total);
+        total = __builtin_amdgcn_readlane(total, 63);
+        // every token may waste one run on rounding: plan for nwaves - T runs
+        ppw = (total + (nwaves - p.T) - 1) / (nwaves - p.T);
+        ppw = ppw < 1 ? 1 : (ppw > LI_MAX_PAIRS_PER_WAVE ? LI_MAX_PAIRS_PER_WAVE : ppw);
+        int base = 0;                     // runs of all tokens before row i of the token table
+        int found = -1;                   // token of this wave's run << 16 | run index... kept separately below
+        int found_run = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int runs = (pairs[i] + ppw - 1) / ppw;
+            const int incl = (int)wave_incl_scan((uint32_t)runs);
+            const int start = base + incl - runs;
+            if (gw >= start && gw < start + runs) { found = l + 64 * i; found_run = gw - start; }
+            base += __builtin_amdgcn_readlane(incl, 63);
+        }
+        const unsigned long long hit = __ballot(found >= 0);
+        if (hit == 0ull) return;          // more waves than runs
+        const int src = __ffsll((long long)hit) - 1;
+        t = __builtin_amdgcn_readlane(found, src);
+        key0 = __builtin_amdgcn_readlane(found_run, src) * (ppw * 64);
+    } else {
+        t = blockIdx.y;
+        ppw = p.ppw;
+        key0 = (blockIdx.x * 4 + w) * (ppw * 64);
+    }
+    const int b = t / p.S1;
+    int cur = p.act[b];
+    cur = cur < 0 ? 0 : (cur > cap ? cap : cur);
     if (key0 >= cur) return;
     int npair = (cur - key0 + 63) >> 6;
-    npair = npair > p.ppw ? p.ppw : npair;
+    npair = npair > ppw ? ppw : npair;
     const int last_blk = ((cur + 31) >> 5) - 1;                  // last 32-key block holding a valid key
 
     // First cache row of every 32-key block of this wave's run, looked up once: lane i holds the row of
@@ -529,58 +622,6 @@ __device__ __forceinline__ unsigned long long order_word(const float score, cons
     return ((unsigned long long)score_key(score) << 32) | (uint32_t)(~pos);
 }
 
-// Wave-wide scan and reductions on DPP (no LDS traffic).  row_shr:n moves a value n lanes up inside
-// its row of 16, row_bcast15/31 carry the last lane of a row / of the lower half-wave upward; lanes
-// without a source keep the identity passed as the old value.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t dpp_u32(const uint32_t identity, const uint32_t v)
-{
-    return (uint32_t)__builtin_amdgcn_update_dpp((int)identity, (int)v, CTRL, ROW_MASK, 0xf, false);
-}
-
-// inclusive prefix sum over the 64 lanes
-__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v)
-{
-    v += dpp_u32<0x111, 0xf>(0u, v);
-    v += dpp_u32<0x112, 0xf>(0u, v);
-    v += dpp_u32<0x114, 0xf>(0u, v);
-    v += dpp_u32<0x118, 0xf>(0u, v);
-    v += dpp_u32<0x142, 0xa>(0u, v);
-    v += dpp_u32<0x143, 0xc>(0u, v);
-    return v;
-}
-
-template <typename Op>
-__device__ __forceinline__ uint32_t wave_reduce_bits(uint32_t v, const uint32_t identity, Op op)
-{
-    v = op(v, dpp_u32<0x111, 0xf>(identity, v));
-    v = op(v, dpp_u32<0x112, 0xf>(identity, v));
-    v = op(v, dpp_u32<0x114, 0xf>(identity, v));
-    v = op(v, dpp_u32<0x118, 0xf>(identity, v));
-    v = op(v, dpp_u32<0x142, 0xa>(identity, v));
-    v = op(v, dpp_u32<0x143, 0xc>(identity, v));
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);     // lane 63 holds the reduction of all lanes
-}
-
-__device__ __forceinline__ float wave_min(const float x)
-{
-    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0x7f800000u, [](uint32_t a, uint32_t b) {
-        return __float_as_uint(fminf(__uint_as_float(a), __uint_as_float(b)));
-    }));
-}
-
-__device__ __forceinline__ float wave_max(const float x)
-{
-    return __uint_as_float(wave_reduce_bits(__float_as_uint(x), 0xff800000u, [](uint32_t a, uint32_t b) {
-        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
-    }));
-}
-
-__device__ __forceinline__ uint32_t wave_max_u32(const uint32_t x)
-{
-    return wave_reduce_bits(x, 0u, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
-}
-
 // score whose order-preserving image is key (the inverse of score_key)
 __device__ __forceinline__ float key_score(const uint32_t key)
 {
@@ -904,8 +945,14 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_stream_kernel(const LiP
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream)
 {
-    const unsigned gx = (unsigned)((p.score_stride + 4 * p.ppw * 64 - 1) / (4 * p.ppw * 64));
-    const dim3 grid(gx, (unsigned)p.T), block(256);
+    const dim3 block(256);
+    dim3 grid;
+    if (p.balanced) {
+        grid = dim3((unsigned)p.score_wgs);
+    } else {
+        const unsigned gx = (unsigned)((p.score_stride + 4 * p.ppw * 64 - 1) / (4 * p.ppw * 64));
+        grid = dim3(gx, (unsigned)p.T);
+    }
     if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
     else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP16>, grid, block, 0, stream, p);
     else hipLaunchKernelGGL(li_score_kernel<PTO_DT_BF16>, grid, block, 0, stream, p);
