@@ -1,0 +1,82 @@
+"""The benchmark configurations at their full sizes on the GPU: the chained path of configuration 2
+(indexer -> attention), configuration 3 (two query tokens per sequence) and configuration 4 (a 4096-token
+prefill), against the C statement of the goldens and through properties that hold at any size."""
+import pytest
+import torch
+
+import pypto_amd
+from pypto_amd.synthetic import config_lengths, gen_indexer_inputs, gen_sfa_inputs
+from pypto_amd.utils import attention_error_stats
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_REL = 2e-2, 5e-3
+DEV = "cuda:0"
+
+
+def run_sfa(inp, topk_indices=None):
+    d = inp.to(torch.device(DEV))
+    out = torch.full([inp.b, inp.s1, inp.n_q, 512], float("nan"), dtype=torch.bfloat16, device=DEV)
+    ti = d.topk_indices if topk_indices is None else topk_indices
+    pypto_amd.sparse_flash_attention_quant_d(d.query_nope, d.query_rope, d.key_nope_2d, d.key_rope_2d,
+                                             d.k_nope_scales, ti, d.block_table, d.kv_act_seqs, out, inp.n_q, 1,
+                                             inp.softmax_scale, inp.topk, inp.block_size, inp.max_blocknum_perbatch,
+                                             None)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def golden(c_oracle, inp, topk_indices=None):
+    ti = inp.topk_indices if topk_indices is None else topk_indices
+    return c_oracle.sfa_quant(inp.query_nope, inp.query_rope, inp.key_nope_2d, inp.key_rope_2d, inp.k_nope_scales, ti,
+                              inp.block_table, inp.kv_act_seqs, inp.b, inp.s1, inp.n_q, inp.topk, inp.block_size,
+                              inp.softmax_scale, s2_tile=0)
+
+
+def check(out, ref, what):
+    assert not torch.isnan(out).any(), f"{what}: NaN in output"
+    max_abs, mean_rel = attention_error_stats(out, ref)
+    print(f"{what}: max_abs={max_abs:.4g} mean_rel={mean_rel:.4g}", flush=True)
+    assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, (what, max_abs, mean_rel)
+
+
+def test_config2_chain_indexer_then_attention(c_oracle):
+    """B=32, KV 8192..65536: the indexer's selection must equal the golden's bit for bit, and the attention
+    over it must match the golden within tolerance."""
+    B, K = 32, 2048
+    lengths = config_lengths(2, seed=2)
+    li = gen_indexer_inputs(B, 1, lengths, selected_count=K, seed=2, variant="fp32")
+    sfa = gen_sfa_inputs(B, 1, 128, lengths, topk=K, seed=3, block_table=li.block_table, block_num=li.block_num,
+                         topk_indices=torch.zeros([B, K], dtype=torch.int32))
+    d = li.to(torch.device(DEV))
+    pypto_amd.lightning_indexer_decode(d.idx_query, d.idx_query_scale, d.idx_key_cache, d.idx_key_scale, d.idx_weight,
+                                       d.act_seq_key, d.block_table, d.topk_res, None, None, K)
+    torch.cuda.synchronize()
+    want = c_oracle.li_decode(li.idx_query, li.idx_query_scale, li.idx_key_cache, li.idx_key_scale, li.idx_weight,
+                              li.act_seq_key, li.block_table, K)
+    got = d.topk_res.cpu()
+    assert torch.equal(got, want), f"{int((got != want).sum())} index mismatches"
+    sel = d.topk_res.reshape(B, K).contiguous()
+    out = run_sfa(sfa, topk_indices=sel)
+    check(out, golden(c_oracle, sfa, topk_indices=sel.cpu()), "cfg2 chain")
+
+
+def test_config3_two_query_tokens_per_sequence(c_oracle):
+    """B=64, S1=2, KV 4096..32768: causal effective lengths, every row against the golden."""
+    lengths = config_lengths(3, seed=3)
+    inp = gen_sfa_inputs(64, 2, 128, lengths, topk=2048, seed=4)
+    out = run_sfa(inp)
+    check(out, golden(c_oracle, inp), "cfg3")
+
+
+def test_config4_prefill_4096_tokens(c_oracle):
+    """B=1, S1=4096, KV 4096: row s sees min(s + 1, 2048) keys.  Every row against the golden; the first
+    row, which sees one key, must be that key's de-quantised value row exactly."""
+    inp = gen_sfa_inputs(1, 4096, 128, config_lengths(4), topk=2048, seed=5)
+    out = run_sfa(inp)
+    # row 0: one key (position 0): out = bf16(int8 * scale) of its cache row, for every head
+    phys = int(inp.block_table[0, 0]) * inp.block_size
+    v = (inp.key_nope_2d[phys].float().reshape(4, 128) * inp.k_nope_scales[phys].reshape(4, 1)).reshape(512)
+    v = v.to(torch.bfloat16)
+    assert torch.equal(out[0, 0].view(torch.int16), v.view(torch.int16).expand(128, 512)), "single-key row"
+    check(out, golden(c_oracle, inp), "cfg4")
