@@ -107,6 +107,15 @@ int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *args, size_t *bytes);
 int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
 
 /*
+ * The non-quantized branch of the same operator (key_nope_2d not int8,
+ * sparse_flash_attention_quant_impl.py:149-153 and 199-202 in the reference
+ * example): key_nope_2d is [kv_rows, 512] bf16 and is used as it is,
+ * k_nope_scales is not read (may be NULL).  Everything else as above; the
+ * workspace is the one pto_sfa_quant_workspace_bytes reports.
+ */
+int pto_sfa_bf16kv_launch(const PtoSfaQuantArgs *args, void *hip_stream);
+
+/*
  * The same attention over the packed cache of sparse_attention_antiquant_d
  * (sparse_attention_antiquant_impl.py:45-85 in the reference example; packing
  * deepseekv32_sparse_attention_antiquant.py:258-268):

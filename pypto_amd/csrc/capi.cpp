@@ -126,7 +126,7 @@ PtoSfaQuantArgs unpacked_view(const PtoSaAntiquantArgs *a)
 
 // checked arguments -> kernel parameters -> launch; the cache is given as three (base, row pitch) pairs
 int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const uint8_t *kr, int kr_pitch, const uint8_t *ksc,
-                int ksc_pitch, void *hip_stream)
+                int ksc_pitch, void *hip_stream, bool kn_bf16 = false)
 {
     const SfaPlan pl = sfa_plan(a);
     const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
@@ -142,6 +142,7 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
     p.kn_pitch = kn_pitch;
     p.kr_pitch = kr_pitch;
     p.ksc_pitch = ksc_pitch;
+    p.kn_bf16 = kn_bf16 ? 1 : 0;
     p.topk_idx = a->topk_indices;
     p.bt = a->block_table;
     p.act = a->kv_act_seqs;
@@ -218,6 +219,17 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *a, void *hip_stream)
         return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
     return sfa_enqueue(a, static_cast<const int8_t *>(a->key_nope_2d), 512, static_cast<const uint8_t *>(a->key_rope_2d), 128,
                        static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream);
+}
+
+int pto_sfa_bf16kv_launch(const PtoSfaQuantArgs *a, void *hip_stream)
+{
+    int rc = sfa_check(a);
+    if (rc != PTO_OK) return rc;
+    if (!a->query_nope || !a->query_rope || !a->key_nope_2d || !a->key_rope_2d || !a->topk_indices || !a->block_table ||
+        !a->kv_act_seqs || !a->attention_out)
+        return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
+    return sfa_enqueue(a, static_cast<const int8_t *>(a->key_nope_2d), 1024, static_cast<const uint8_t *>(a->key_rope_2d), 128,
+                       static_cast<const uint8_t *>(a->key_nope_2d), 0, hip_stream, true);
 }
 
 int pto_sa_antiquant_workspace_bytes(const PtoSaAntiquantArgs *a, size_t *bytes)

@@ -120,6 +120,17 @@ PYBIND11_MODULE(_C, m)
               check(pto_sfa_quant_launch(&a, ptr<void>(stream)));
           });
 
+    m.def("sfa_bf16kv_launch",
+          [](std::uintptr_t query_nope, std::uintptr_t query_rope, std::uintptr_t key_nope_2d, std::uintptr_t key_rope_2d,
+             std::uintptr_t topk_indices, std::uintptr_t block_table, std::uintptr_t kv_act_seqs,
+             std::uintptr_t attention_out, std::uintptr_t workspace, size_t workspace_bytes, int64_t b, int64_t s1,
+             int64_t nq, int64_t n_kv, int64_t topk, int64_t block_size, int64_t max_blocknum_perbatch, int64_t kv_rows,
+             double softmax_scale, int num_splits, std::uintptr_t stream) {
+              PtoSfaQuantArgs a = sfa_args(query_nope, query_rope, key_nope_2d, key_rope_2d, 0, topk_indices, block_table,
+                                           kv_act_seqs, attention_out, workspace, workspace_bytes, b, s1, nq, n_kv, topk,
+                                           block_size, max_blocknum_perbatch, kv_rows, softmax_scale, num_splits);
+              check(pto_sfa_bf16kv_launch(&a, ptr<void>(stream)));
+          });
     m.def("sa_antiquant_launch",
           [](std::uintptr_t query_nope, std::uintptr_t query_rope, std::uintptr_t nope_cache, std::uintptr_t topk_indices,
              std::uintptr_t block_table, std::uintptr_t kv_act_seqs, std::uintptr_t attention_out, std::uintptr_t workspace,

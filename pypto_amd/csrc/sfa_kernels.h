@@ -17,6 +17,7 @@ struct SfaParams {
     const uint8_t *kr;        // 64 bf16 rope values
     const uint8_t *ksc;       // 4 fp32 scales, one per 128 latent channels
     int kn_pitch, kr_pitch, ksc_pitch;
+    int kn_bf16;              // the latent part is bf16 (1024 bytes, no scales) instead of int8
     const int32_t *topk_idx;  // [T, topk]
     const int32_t *bt;        // [B, maxblk]
     const int32_t *act;       // [B]

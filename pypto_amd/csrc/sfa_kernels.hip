@@ -115,7 +115,9 @@ __device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
 
 constexpr float RESCALE_TAU = 8.0f;   // log2 units: the reference max moves only when exceeded by 2^8
 
-template <int NW>
+// QUANT: the latent part of a cache row is int8 with four fp32 scales and is de-quantised on the way into
+// LDS; otherwise it is bf16 already (1024 bytes) and travels cache -> LDS tile directly by LDS-DMA.
+template <int NW, bool QUANT>
 __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 {
     // One LDS pool.  Prologue: all 32*NW query heads staged at once (PITCH elements each).  Loop: tile
@@ -258,13 +260,22 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 
     // wave w gathers keys w*KT/NW .. +KT/NW of the tile; within a pass the lower half-wave takes key
     // half*NP + i, so a lane's NP row numbers are one contiguous LDS read
-    auto issue_loads = [&](const int kt) {
-        const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW) + half * NP;
+    auto issue_loads = [&](const int kt, uint16_t *buf) {
+        if (QUANT) {
+            const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW) + half * NP;
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
-            const int row = rtab[i];
-            raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * p.kn_pitch + 16 * col);
-            rsc[i] = *reinterpret_cast<const float *>(p.ksc + (size_t)row * p.ksc_pitch + 4 * (col >> 3));
+            for (int i = 0; i < NP; ++i) {
+                const int row = rtab[i];
+                raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * p.kn_pitch + 16 * col);
+                rsc[i] = *reinterpret_cast<const float *>(p.ksc + (size_t)row * p.ksc_pitch + 4 * (col >> 3));
+            }
+        } else {
+            // one request per key: the 64 lanes' 16-byte pieces are the 1024 bytes of the row, in order
+            const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW);
+#pragma unroll
+            for (int i = 0; i < KT / NW; ++i)
+                dma16(p.kn + (size_t)rtab[i] * p.kn_pitch + 16 * l,
+                      (uint32_t)(uintptr_t)(lds_byte_t *)(buf + (w * (KT / NW) + i) * PITCH));
         }
 #pragma unroll
         for (int i = 0; i < RP; ++i) {
@@ -281,7 +292,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 #pragma unroll
         for (int q = 0; q < PER; ++q) {
             const int hidx = piece * PER + q;
-            if (hidx < HALVES) {
+            if (QUANT && hidx < HALVES) {
                 const int i = hidx >> 1, hh = hidx & 1;
                 const int kl = w * (KT / NW) + half * NP + i;
                 dequant8(raw[i][2 * hh], raw[i][2 * hh + 1], rsc[i], buf + kl * PITCH + 16 * col + 8 * hh);
@@ -303,9 +314,10 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     collect_q(1);
     __syncthreads();                       // row table complete, pool free again
     if (k_begin < k_end) {
-        issue_loads(k_begin);
+        issue_loads(k_begin, tile0);
         store_tile(tile0);
     }
+    if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);     // this wave's direct requests into the tile have landed
     __syncthreads();
     // All global loads issued so far (Q^T fragments, first tile) are complete from here on, so that
     // inside the loop the only outstanding vector-memory operations are the next tile's gather and
@@ -316,7 +328,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     for (int kt = k_begin; kt < k_end; kt += KT, ++it) {
         const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
         uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
-        issue_loads(kt + KT);                    // next tile (or the padding tile): in flight during the products
+        issue_loads(kt + KT, nxt_tile);          // next tile (or the padding tile): in flight during the products
 
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
@@ -415,6 +427,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's direct requests into the next tile have landed
         __syncthreads();
     }
 
@@ -550,10 +563,18 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
 {
     const int rows8 = (p.T + 7) / 8 * 8;
     const unsigned grid = (unsigned)(rows8 * p.hgroups * p.nsplit);
-    switch (p.waves) {
-    case 1: hipLaunchKernelGGL(sfa_decode_kernel<1>, dim3(grid), dim3(64), 0, stream, p); break;
-    case 2: hipLaunchKernelGGL(sfa_decode_kernel<2>, dim3(grid), dim3(128), 0, stream, p); break;
-    default: hipLaunchKernelGGL(sfa_decode_kernel<4>, dim3(grid), dim3(256), 0, stream, p); break;
+    if (p.kn_bf16) {
+        switch (p.waves) {
+        case 1: hipLaunchKernelGGL((sfa_decode_kernel<1, false>), dim3(grid), dim3(64), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL((sfa_decode_kernel<2, false>), dim3(grid), dim3(128), 0, stream, p); break;
+        default: hipLaunchKernelGGL((sfa_decode_kernel<4, false>), dim3(grid), dim3(256), 0, stream, p); break;
+        }
+    } else {
+        switch (p.waves) {
+        case 1: hipLaunchKernelGGL((sfa_decode_kernel<1, true>), dim3(grid), dim3(64), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL((sfa_decode_kernel<2, true>), dim3(grid), dim3(128), 0, stream, p); break;
+        default: hipLaunchKernelGGL((sfa_decode_kernel<4, true>), dim3(grid), dim3(256), 0, stream, p); break;
+        }
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

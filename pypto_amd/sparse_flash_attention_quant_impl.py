@@ -49,26 +49,28 @@ def _launch(query_nope, query_rope, key_nope_2d, key_rope_2d, k_nope_scales, top
     qr = as_torch(query_rope, "query_rope")
     kn = as_torch(key_nope_2d, "key_nope_2d")
     kr = as_torch(key_rope_2d, "key_rope_2d")
-    ks = as_torch(k_nope_scales, "k_nope_scales")
+    quant = kn.dtype == torch.int8                       # else the non-quantized branch (:149-153, :199-202)
+    ks = as_torch(k_nope_scales, "k_nope_scales") if quant or k_nope_scales is not None else None
     ti = as_torch(topk_indices, "topk_indices")
     bt = as_torch(block_table, "block_table")
     act = as_torch(kv_act_seqs, "kv_act_seqs")
     out = as_torch(attention_out, "attention_out")
 
-    tensors = (qn, qr, kn, kr, ks, ti, bt, act, out)
+    tensors = tuple(x for x in (qn, qr, kn, kr, ks, ti, bt, act, out) if x is not None)
     dev = qn.device
     if dev.type != "cuda":
         raise RuntimeError("sparse_flash_attention_quant: tensors must live on the GPU (device type 'cuda' on ROCm)")
     if any(t.device != dev for t in tensors):
         raise RuntimeError("not all tensors are on the same device")   # python/pypto/runtime.py:224-228
 
-    if kn.dtype != torch.int8:
-        raise TypeError("key_nope_2d: only the int8 (quantized) cache is implemented")
+    if kn.dtype not in (torch.int8, torch.bfloat16):
+        raise TypeError(f"key_nope_2d: expected int8 (quantized cache) or bfloat16, got {kn.dtype}")
     _check(qn, "query_nope", torch.bfloat16, 2)
     _check(qr, "query_rope", torch.bfloat16, 2)
-    _check(kn, "key_nope_2d", torch.int8, 2)
+    _check(kn, "key_nope_2d", kn.dtype, 2)
     _check(kr, "key_rope_2d", torch.bfloat16, 2)
-    _check(ks, "k_nope_scales", torch.float32, 2)
+    if quant:
+        _check(ks, "k_nope_scales", torch.float32, 2)
     _check(ti, "topk_indices", torch.int32, 2)
     _check(bt, "block_table", torch.int32, 2)
     _check(act, "kv_act_seqs", torch.int32, 1)
@@ -83,7 +85,7 @@ def _launch(query_nope, query_rope, key_nope_2d, key_rope_2d, k_nope_scales, top
         raise ValueError("query_nope/query_rope: first dimension must be b*s1*nq")
     s1 = qn.shape[0] // (b * nq)
     rows = kn.shape[0]
-    if kn.shape[1] != KV_LORA_RANK or tuple(kr.shape) != (rows, ROPE_DIM) or tuple(ks.shape) != (rows, 4):
+    if kn.shape[1] != KV_LORA_RANK or tuple(kr.shape) != (rows, ROPE_DIM) or (quant and tuple(ks.shape) != (rows, 4)):
         raise ValueError("key_nope_2d/key_rope_2d/k_nope_scales: expected [rows,512], [rows,64], [rows,4]")
     if tuple(ti.shape) != (b * s1, n_kv * topk):
         raise ValueError(f"topk_indices: expected shape {(b * s1, n_kv * topk)}, got {tuple(ti.shape)}")
@@ -98,9 +100,14 @@ def _launch(query_nope, query_rope, key_nope_2d, key_rope_2d, k_nope_scales, top
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)   # caching allocator, stream-ordered
     stream = torch.cuda.current_stream(dev).cuda_stream
     with torch.cuda.device(dev):
-        C.sfa_quant_launch(qn.data_ptr(), qr.data_ptr(), kn.data_ptr(), kr.data_ptr(), ks.data_ptr(), ti.data_ptr(),
-                           bt.data_ptr(), act.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, b, s1, nq, n_kv,
-                           topk, block_size, bt_cols, rows, float(softmax_scale), int(num_splits), stream)
+        if quant:
+            C.sfa_quant_launch(qn.data_ptr(), qr.data_ptr(), kn.data_ptr(), kr.data_ptr(), ks.data_ptr(), ti.data_ptr(),
+                               bt.data_ptr(), act.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, b, s1, nq, n_kv,
+                               topk, block_size, bt_cols, rows, float(softmax_scale), int(num_splits), stream)
+        else:
+            C.sfa_bf16kv_launch(qn.data_ptr(), qr.data_ptr(), kn.data_ptr(), kr.data_ptr(), ti.data_ptr(), bt.data_ptr(),
+                                act.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, b, s1, nq, n_kv, topk,
+                                block_size, bt_cols, rows, float(softmax_scale), int(num_splits), stream)
     return None
 
 

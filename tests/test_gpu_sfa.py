@@ -174,3 +174,33 @@ def test_packed_cache_operator(n_q, b, s1, act, topk, entry):
                                       inp.block_size, inp.softmax_scale, inp.topk)
     check(out, ref, f"packed nq={n_q} b={b} s1={s1} act={act} topk={topk}")
     assert torch.equal(out.view(torch.int16), run_op(inp, entry=entry).view(torch.int16))
+
+
+# ------------------------------------------------------------------ non-quantized (bf16) latent cache
+
+@pytest.mark.parametrize("n_q,b,s1,act,topk", [
+    (128, 2, 1, [5000, 3000], 2048),
+    (16, 1, 1, [4096], 256),
+    (64, 2, 2, [300, 70], 128),
+])
+def test_bf16_latent_cache_branch(n_q, b, s1, act, topk):
+    """key_nope_2d in bf16, no scales: against the golden's non-quantized branch, and -- fed with exactly
+    the values the int8 cache de-quantises to -- bit-identical to the quantized operator."""
+    from oracle import sfa_oracle as so
+    inp = gen_sfa_inputs(b, s1, n_q, act, topk=topk, seed=23 + n_q)
+    kn_bf16 = so.dequant_kn(inp.key_nope_2d, inp.k_nope_scales)
+    assert kn_bf16.dtype == torch.bfloat16
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    out = torch.full([inp.b, inp.s1, inp.n_q, 512], float("nan"), dtype=torch.bfloat16, device=dev)
+    ret = pypto_amd.sparse_flash_attention_quant_d(d.query_nope, d.query_rope, kn_bf16.to(dev), d.key_rope_2d, None,
+                                                   d.topk_indices, d.block_table, d.kv_act_seqs, out, inp.n_q, 1,
+                                                   inp.softmax_scale, inp.topk, inp.block_size,
+                                                   inp.max_blocknum_perbatch, None)
+    assert ret is None
+    torch.cuda.synchronize()
+    out = out.cpu()
+    ref = so.sfa_single_pass(inp.q_bsnd(), kn_bf16, inp.key_rope_2d, None, inp.topk_indices, inp.block_table,
+                             inp.actual_seq, inp.block_size, inp.softmax_scale, inp.topk, is_kn_quant=False)
+    check(out, ref, f"bf16 cache nq={n_q} b={b} s1={s1}")
+    assert torch.equal(out.view(torch.int16), run_op(inp).view(torch.int16))
