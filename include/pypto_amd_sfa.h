@@ -30,6 +30,11 @@
  *       the device execution of lightning_indexer_decode
  *       (examples/models/deepseek_v32_exp/lightning_indexer_quant_impl.py:315-346),
  *       same dispatch point.
+ *   pto_li_prolog_quant_launch
+ *       the device execution of lightning_indexer_prolog_quant
+ *       (examples/models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:507-562),
+ *       same dispatch point: the projection stage that produces the indexer's
+ *       int8 query, per-head weights and the new int8 key rows of the paged cache.
  *   pto_*_workspace_bytes
  *       the workspace query the reference runtime performs before a launch
  *       (python/pypto/runtime.py:151-152, GetWorkSpaceSize).
@@ -202,6 +207,72 @@ typedef struct PtoLiDecodeArgs {
 
 int pto_li_decode_workspace_bytes(const PtoLiDecodeArgs *args, size_t *bytes);
 int pto_li_decode_launch(const PtoLiDecodeArgs *args, void *hip_stream);
+
+/*
+ * Lightning-indexer prolog, quantized (lightning_indexer_prolog_quant_impl.py:325-504
+ * in the reference example; torch golden
+ * deepseekv32_lightning_indexer_prolog_quant.py:216-281):
+ *
+ *   x              [t, h]                        bf16
+ *   q_norm         [t, q_lora_rank]              int8
+ *   q_norm_scale   [t, 1]                        fp32
+ *   w_qb           [q_lora_rank, n_heads*128]    int8   row-major (the reference passes
+ *                                                       its NPU fractal form of this matrix)
+ *   w_qb_scale     [n_heads*128, 1]              fp32
+ *   wk             [h, 128]                      bf16   row-major
+ *   w_proj         [h, n_heads]                  bf16   row-major
+ *   ln_gamma_k, ln_beta_k  [128]                 bf16
+ *   cos_idx_rope, sin_idx_rope  [t, 64]          bf16
+ *   hadamard_q, hadamard_k      [128, 128]       bf16
+ *   k_cache        [block_num, block_size, 1, 128]  int8   rows k_cache_index[i] rewritten
+ *   k_cache_scale  [block_num, block_size, 1, 1]    fp16   same rows
+ *   k_cache_index  [t]                           int64  physical cache row of each token
+ *   q_int8         [t, n_heads, 128]             int8   written
+ *   q_scale        [t, n_heads, 1]               fp16   written
+ *   weights        [t, n_heads]                  fp16   written
+ *
+ * Every fp32 sum has a fixed order, so results are reproducible bit for bit:
+ * sums over h in blocks of 64 (ascending inside a block, blocks ascending), the
+ * 128-term Hadamard sums ascending, the layer-norm means as balanced trees over
+ * neighbouring channels.  A row whose values are all zero quantises to zeros with
+ * scale 0.  Cache indices outside [0, cache_rows) are skipped.
+ *
+ * Constraints: head_dim 128, rope 64, 1 <= n_heads <= 64, q_lora_rank in
+ * {512, 1024, 1536}, h a positive multiple of 64, t >= 1.
+ */
+typedef struct PtoLiPrologQuantArgs {
+    const void *x;
+    const int8_t *q_norm;
+    const float *q_norm_scale;
+    const int8_t *w_qb;
+    const float *w_qb_scale;
+    const void *wk;
+    const void *w_proj;
+    const void *ln_gamma_k;
+    const void *ln_beta_k;
+    const void *cos_idx_rope;
+    const void *sin_idx_rope;
+    const void *hadamard_q;
+    const void *hadamard_k;
+    int8_t *k_cache;
+    void *k_cache_scale;
+    const int64_t *k_cache_index;
+    int8_t *q_int8;
+    void *q_scale;
+    void *weights;
+    void *workspace;
+    size_t workspace_bytes;
+    int64_t t;
+    int64_t h;
+    int64_t q_lora_rank;
+    int64_t n_heads;
+    int64_t cache_rows;   /* block_num * block_size */
+    float eps;            /* layer-norm epsilon (attrs.eps) */
+    int32_t reserved;
+} PtoLiPrologQuantArgs;
+
+int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *args, size_t *bytes);
+int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *args, void *hip_stream);
 
 /* Thread-local description of the last error on this thread ("" if none). */
 const char *pto_last_error(void);

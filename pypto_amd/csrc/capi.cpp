@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "li_kernels.h"
+#include "lip_kernels.h"
 #include "sfa_kernels.h"
 
 namespace {
@@ -192,6 +193,31 @@ size_t li_ws_bytes(const PtoLiDecodeArgs *a)
     return (size_t)a->t * stride * sizeof(float);
 }
 
+int lip_check(const PtoLiPrologQuantArgs *a)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "li_prolog: args is NULL");
+    if (a->t < 1 || a->t > (1ll << 20)) return fail(PTO_E_INVALID_ARG, "li_prolog: t must be in [1, 2^20]");
+    if (a->n_heads < 1 || a->n_heads > pto::LIP_MAX_HEADS)
+        return fail(PTO_E_INVALID_ARG, "li_prolog: n_heads must be in [1, %d] (got %lld)", pto::LIP_MAX_HEADS, (long long)a->n_heads);
+    if (a->q_lora_rank != 512 && a->q_lora_rank != 1024 && a->q_lora_rank != 1536)
+        return fail(PTO_E_INVALID_ARG, "li_prolog: q_lora_rank must be 512, 1024 or 1536 (got %lld)", (long long)a->q_lora_rank);
+    if (a->h < pto::LIP_XBLOCK || a->h % pto::LIP_XBLOCK != 0 || a->h > (1ll << 20))
+        return fail(PTO_E_INVALID_ARG, "li_prolog: h must be a positive multiple of %d (got %lld)", pto::LIP_XBLOCK, (long long)a->h);
+    if (a->cache_rows < 1 || a->cache_rows > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "li_prolog: cache_rows out of range");
+    if (!std::isfinite(a->eps) || a->eps < 0) return fail(PTO_E_INVALID_ARG, "li_prolog: eps must be finite and >= 0");
+    return PTO_OK;
+}
+
+// [4 partial int32 projections | block sums over the hidden axis]
+size_t lip_qpart_bytes(const PtoLiPrologQuantArgs *a)
+{
+    return (size_t)pto::LIP_KSPLIT * a->t * a->n_heads * pto::LIP_DIM * sizeof(int32_t);
+}
+size_t lip_ws_bytes(const PtoLiPrologQuantArgs *a)
+{
+    return lip_qpart_bytes(a) + (size_t)(a->h / pto::LIP_XBLOCK) * a->t * pto::LIP_XCOLS * sizeof(float);
+}
+
 }  // namespace
 
 extern "C" {
@@ -309,6 +335,68 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     }
     hipError_t e = pto::li_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
+int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *a, size_t *bytes)
+{
+    if (!bytes) return fail(PTO_E_INVALID_ARG, "li_prolog: bytes is NULL");
+    int rc = lip_check(a);
+    if (rc != PTO_OK) return rc;
+    *bytes = lip_ws_bytes(a);
+    return PTO_OK;
+}
+
+int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
+{
+    int rc = lip_check(a);
+    if (rc != PTO_OK) return rc;
+    if (!a->x || !a->q_norm || !a->q_norm_scale || !a->w_qb || !a->w_qb_scale || !a->wk || !a->w_proj || !a->ln_gamma_k ||
+        !a->ln_beta_k || !a->cos_idx_rope || !a->sin_idx_rope || !a->hadamard_q || !a->hadamard_k || !a->k_cache ||
+        !a->k_cache_scale || !a->k_cache_index || !a->q_int8 || !a->q_scale || !a->weights)
+        return fail(PTO_E_INVALID_ARG, "li_prolog: a tensor pointer is NULL");
+    const size_t need = lip_ws_bytes(a);
+    if (!a->workspace || a->workspace_bytes < need)
+        return fail(PTO_E_WORKSPACE, "li_prolog: workspace of %zu bytes required, %zu given", need,
+                    a->workspace ? a->workspace_bytes : (size_t)0);
+    const void *aligned[] = {a->x, a->q_norm, a->q_norm_scale, a->w_qb, a->w_qb_scale, a->wk, a->ln_gamma_k, a->ln_beta_k,
+                             a->cos_idx_rope, a->sin_idx_rope, a->hadamard_q, a->hadamard_k, a->k_cache, a->q_int8, a->workspace};
+    for (const void *ptr : aligned)
+        if (reinterpret_cast<uintptr_t>(ptr) & 15)
+            return fail(PTO_E_INVALID_ARG, "li_prolog: tensor and workspace pointers must be 16-byte aligned");
+
+    pto::LipParams p;
+    p.x = static_cast<const uint16_t *>(a->x);
+    p.q_norm = a->q_norm;
+    p.q_norm_scale = a->q_norm_scale;
+    p.w_qb = a->w_qb;
+    p.w_qb_scale = a->w_qb_scale;
+    p.wk = static_cast<const uint16_t *>(a->wk);
+    p.w_proj = static_cast<const uint16_t *>(a->w_proj);
+    p.gamma = static_cast<const uint16_t *>(a->ln_gamma_k);
+    p.beta = static_cast<const uint16_t *>(a->ln_beta_k);
+    p.cos = static_cast<const uint16_t *>(a->cos_idx_rope);
+    p.sin = static_cast<const uint16_t *>(a->sin_idx_rope);
+    p.hq = static_cast<const uint16_t *>(a->hadamard_q);
+    p.hk = static_cast<const uint16_t *>(a->hadamard_k);
+    p.k_cache = a->k_cache;
+    p.k_cache_scale = static_cast<uint16_t *>(a->k_cache_scale);
+    p.k_cache_index = reinterpret_cast<const long long *>(a->k_cache_index);
+    p.q_int8 = a->q_int8;
+    p.q_scale = static_cast<uint16_t *>(a->q_scale);
+    p.weights = static_cast<uint16_t *>(a->weights);
+    p.qpart = static_cast<int32_t *>(a->workspace);
+    p.xpart = reinterpret_cast<float *>(static_cast<char *>(a->workspace) + lip_qpart_bytes(a));
+    p.cache_rows = a->cache_rows;
+    p.T = (int)a->t;
+    p.h = (int)a->h;
+    p.q_lora = (int)a->q_lora_rank;
+    p.n_heads = (int)a->n_heads;
+    p.eps = a->eps;
+    p.w_mul0 = (float)std::pow((double)a->n_heads, -0.5);
+    p.w_mul1 = (float)std::pow((double)pto::LIP_DIM, -0.5);
+    hipError_t e = pto::lip_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
 }
 

@@ -45,4 +45,24 @@ __device__ __forceinline__ s16x4 lds_read_tr16(const uint16_t *p)
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p));
 }
 
+typedef __attribute__((address_space(3))) uint8_t lds_byte_t;
+
+// One LDS-DMA request: lane i's 16 bytes at base + lane_off land at lds_dst + 16*i.  base and lds_dst
+// are wave-uniform.  Written as assembly so that the compiler tracks none of these requests: an
+// explicit vmcnt wait follows them.
+__device__ __forceinline__ void dma16_base(const void *base, const uint32_t lane_off, const uint32_t lds_dst)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    const uint64_t ub = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b) |
+                        ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(ub), "s"(dst) : "memory", "m0");
+}
+// the same with a full address per lane
+__device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
+}
+
 }  // namespace pto

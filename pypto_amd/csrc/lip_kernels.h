@@ -1,0 +1,45 @@
+// Launch parameters of the lightning-indexer prolog kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+constexpr int LIP_DIM = 128;        // channels per indexer head
+constexpr int LIP_ROPE = 64;        // leading channels that are rotated
+constexpr int LIP_KSPLIT = 4;       // workgroups that share the reduction axis of the query projection
+constexpr int LIP_XBLOCK = 64;      // block length of the fixed-order sums over the hidden axis
+constexpr int LIP_XCOLS = 192;      // columns of one partial row: 128 key channels, then up to 64 head weights
+constexpr int LIP_MAX_HEADS = 64;
+constexpr int LIP_MAX_QLORA = 2048; // the quarter tile of w_qb (q_lora_rank/4 rows of 128 bytes) must fit in 64 KiB of LDS
+
+struct LipParams {
+    const uint16_t *x;           // [T, h] bf16
+    const int8_t *q_norm;        // [T, q_lora]
+    const float *q_norm_scale;   // [T]
+    const int8_t *w_qb;          // [q_lora, n_heads*128]
+    const float *w_qb_scale;     // [n_heads*128]
+    const uint16_t *wk;          // [h, 128] bf16
+    const uint16_t *w_proj;      // [h, n_heads] bf16
+    const uint16_t *gamma;       // [128] bf16
+    const uint16_t *beta;        // [128] bf16
+    const uint16_t *cos;         // [T, 64] bf16
+    const uint16_t *sin;         // [T, 64] bf16
+    const uint16_t *hq;          // [128, 128] bf16
+    const uint16_t *hk;          // [128, 128] bf16
+    int8_t *k_cache;             // [cache_rows, 128]
+    uint16_t *k_cache_scale;     // [cache_rows] fp16
+    const long long *k_cache_index;  // [T]
+    int8_t *q_int8;              // [T, n_heads, 128]
+    uint16_t *q_scale;           // [T, n_heads] fp16
+    uint16_t *weights;           // [T, n_heads] fp16
+    int32_t *qpart;              // workspace [LIP_KSPLIT, T, n_heads*128]
+    float *xpart;                // workspace [h/64, T, LIP_XCOLS]
+    long long cache_rows;
+    int T, h, q_lora, n_heads;
+    float eps, w_mul0, w_mul1;   // weights = fp16((bf16(x.w_proj) * w_mul0) * w_mul1)
+};
+
+hipError_t lip_launch(const LipParams &p, hipStream_t stream);
+
+}  // namespace pto

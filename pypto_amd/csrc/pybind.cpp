@@ -180,4 +180,53 @@ PYBIND11_MODULE(_C, m)
                                           block_num, block_size, max_blocknum_perbatch, selected_count, q_dt, k_dt, w_dt);
               check(pto_li_decode_launch(&a, ptr<void>(stream)));
           });
+
+    m.def("li_prolog_quant_workspace_bytes", [](int64_t t, int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows) {
+        PtoLiPrologQuantArgs a{};
+        a.t = t;
+        a.h = h;
+        a.q_lora_rank = q_lora_rank;
+        a.n_heads = n_heads;
+        a.cache_rows = cache_rows;
+        size_t bytes = 0;
+        check(pto_li_prolog_quant_workspace_bytes(&a, &bytes));
+        return bytes;
+    });
+    m.def("li_prolog_quant_launch",
+          [](std::uintptr_t x, std::uintptr_t q_norm, std::uintptr_t q_norm_scale, std::uintptr_t w_qb, std::uintptr_t w_qb_scale,
+             std::uintptr_t wk, std::uintptr_t w_proj, std::uintptr_t ln_gamma_k, std::uintptr_t ln_beta_k,
+             std::uintptr_t cos_idx_rope, std::uintptr_t sin_idx_rope, std::uintptr_t hadamard_q, std::uintptr_t hadamard_k,
+             std::uintptr_t k_cache, std::uintptr_t k_cache_scale, std::uintptr_t k_cache_index, std::uintptr_t q_int8,
+             std::uintptr_t q_scale, std::uintptr_t weights, std::uintptr_t workspace, size_t workspace_bytes, int64_t t,
+             int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows, double eps, std::uintptr_t stream) {
+              PtoLiPrologQuantArgs a{};
+              a.x = ptr<const void>(x);
+              a.q_norm = ptr<const int8_t>(q_norm);
+              a.q_norm_scale = ptr<const float>(q_norm_scale);
+              a.w_qb = ptr<const int8_t>(w_qb);
+              a.w_qb_scale = ptr<const float>(w_qb_scale);
+              a.wk = ptr<const void>(wk);
+              a.w_proj = ptr<const void>(w_proj);
+              a.ln_gamma_k = ptr<const void>(ln_gamma_k);
+              a.ln_beta_k = ptr<const void>(ln_beta_k);
+              a.cos_idx_rope = ptr<const void>(cos_idx_rope);
+              a.sin_idx_rope = ptr<const void>(sin_idx_rope);
+              a.hadamard_q = ptr<const void>(hadamard_q);
+              a.hadamard_k = ptr<const void>(hadamard_k);
+              a.k_cache = ptr<int8_t>(k_cache);
+              a.k_cache_scale = ptr<void>(k_cache_scale);
+              a.k_cache_index = ptr<const int64_t>(k_cache_index);
+              a.q_int8 = ptr<int8_t>(q_int8);
+              a.q_scale = ptr<void>(q_scale);
+              a.weights = ptr<void>(weights);
+              a.workspace = ptr<void>(workspace);
+              a.workspace_bytes = workspace_bytes;
+              a.t = t;
+              a.h = h;
+              a.q_lora_rank = q_lora_rank;
+              a.n_heads = n_heads;
+              a.cache_rows = cache_rows;
+              a.eps = static_cast<float>(eps);
+              check(pto_li_prolog_quant_launch(&a, ptr<void>(stream)));
+          });
 }

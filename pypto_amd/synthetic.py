@@ -11,6 +11,9 @@ the reference tree):
   shapes and layouts of the operator inputs; index rows are a random subset of
   the valid positions, or ``arange`` when fewer than ``topk`` exist)
 * ``gen_indexer_inputs`` ...lightning_indexer_quant.py:119-181
+* ``gen_indexer_prolog_inputs`` ...deepseekv32_lightning_indexer_prolog_quant.py:100-153
+  (value ranges, tensor names and shapes; ``cache_index`` names the last ``s1``
+  positions of every sequence, :76-84)
 
 Unlike the reference (global ``torch.manual_seed`` plus an unseeded
 ``np.random.permutation``) every generator here draws from an explicit
@@ -205,6 +208,88 @@ def gen_indexer_inputs(b: int, s1: int, act_seq: Sequence[int], selected_count: 
                          act_seq=act, idx_query=q, idx_query_scale=qs, idx_key_cache=k, idx_key_scale=ks,
                          idx_weight=w, act_seq_key=torch.tensor(act, dtype=torch.int32), block_table=block_table,
                          topk_res=torch.zeros([t, 1, selected_count], dtype=torch.int32))
+
+
+@dataclass
+class IndexerPrologInputs:
+    b: int
+    s1: int
+    block_size: int
+    block_num: int
+    act_seq: List[int]
+    x: torch.Tensor              # [T, h]                 bf16
+    q_norm: torch.Tensor         # [T, q_lora_rank]       int8
+    q_norm_scale: torch.Tensor   # [T, 1]                 fp32
+    w_qb: torch.Tensor           # [q_lora_rank, N*128]   int8
+    w_qb_scale: torch.Tensor     # [N*128, 1]             fp32
+    wk: torch.Tensor             # [h, 128]               bf16
+    w_proj: torch.Tensor         # [h, N]                 bf16
+    ln_gamma_k: torch.Tensor     # [128]                  bf16
+    ln_beta_k: torch.Tensor      # [128]                  bf16
+    cos_idx_rope: torch.Tensor   # [T, 64]                bf16
+    sin_idx_rope: torch.Tensor   # [T, 64]                bf16
+    hadamard_q: torch.Tensor     # [128, 128]             bf16
+    hadamard_k: torch.Tensor     # [128, 128]             bf16
+    k_cache: torch.Tensor        # [NB, bs, 1, 128]       int8   (updated in place)
+    k_cache_scale: torch.Tensor  # [NB, bs, 1, 1]         fp16   (updated in place)
+    k_cache_index: torch.Tensor  # [T]                    int64
+    block_table: torch.Tensor    # [B, MB]                int32
+
+    def input_tensors(self):
+        return (self.x, self.q_norm, self.q_norm_scale, self.w_qb, self.w_qb_scale, self.wk, self.w_proj,
+                self.ln_gamma_k, self.ln_beta_k, self.cos_idx_rope, self.sin_idx_rope, self.hadamard_q,
+                self.hadamard_k, self.k_cache, self.k_cache_scale, self.k_cache_index)
+
+    def to(self, device) -> "IndexerPrologInputs":
+        kw = dict(self.__dict__)
+        for k, v in kw.items():
+            if isinstance(v, torch.Tensor):
+                kw[k] = v.to(device)
+        return IndexerPrologInputs(**kw)
+
+
+def gen_indexer_prolog_inputs(b: int, s1: int, act_seq: Sequence[int], seed: int = 0, h: int = 7168,
+                              q_lora_rank: int = 1536, n_heads: int = IDX_HEADS, head_dim: int = IDX_DIM,
+                              rope_dim: int = ROPE_DIM, block_size: int = BLOCK_SIZE,
+                              affine_ln: bool = False) -> IndexerPrologInputs:
+    """Value ranges of the reference generator: x, weights and Hadamard matrices uniform in (-1, 1) bf16,
+    int8 operands uniform over the full range, scales uniform in (-1, 1), cos/sin of uniform angles, cache
+    filled with random rows.  ``affine_ln`` draws gamma/beta at random instead of the reference's 1/0."""
+    g = torch.Generator().manual_seed(seed)
+    act = [int(a) for a in act_seq]
+    t = b * s1
+    bf = torch.bfloat16
+
+    def uni(shape, dtype):
+        return (torch.rand(shape, generator=g, dtype=torch.float32) * 2 - 1).to(dtype)
+
+    x = uni([t, h], bf)
+    q_norm = torch.randint(-128, 128, [t, q_lora_rank], generator=g, dtype=torch.int8)
+    q_norm_scale = uni([t, 1], torch.float32)
+    w_qb = torch.randint(-128, 128, [q_lora_rank, n_heads * head_dim], generator=g, dtype=torch.int8)
+    w_qb_scale = uni([n_heads * head_dim, 1], torch.float32)
+    wk = uni([h, head_dim], bf)
+    w_proj = uni([h, n_heads], bf)
+    if affine_ln:
+        gamma, beta = uni([head_dim], bf), uni([head_dim], bf)
+    else:
+        gamma, beta = torch.ones([head_dim], dtype=bf), torch.zeros([head_dim], dtype=bf)
+    ang = torch.rand([t, rope_dim], generator=g, dtype=torch.float32) * (2 * math.pi)
+    cos, sin = torch.cos(ang).to(bf), torch.sin(ang).to(bf)
+    hq, hk = uni([head_dim, head_dim], bf), uni([head_dim, head_dim], bf)
+    block_num, table = gen_block_table(act, block_size, g, shuffle=True)
+    k_cache = torch.randint(-128, 128, [block_num, block_size, 1, head_dim], generator=g, dtype=torch.int8)
+    k_cache_scale = uni([block_num, block_size, 1, 1], torch.float16)
+    idx = torch.empty([b, s1], dtype=torch.int64)
+    for i in range(b):
+        for j in range(s1):
+            pos = act[i] - s1 + j
+            idx[i, j] = int(table[i, pos // block_size]) * block_size + pos % block_size
+    return IndexerPrologInputs(b=b, s1=s1, block_size=block_size, block_num=block_num, act_seq=act, x=x,
+                               q_norm=q_norm, q_norm_scale=q_norm_scale, w_qb=w_qb, w_qb_scale=w_qb_scale,
+                               wk=wk, w_proj=w_proj, ln_gamma_k=gamma, ln_beta_k=beta, cos_idx_rope=cos,
+                               sin_idx_rope=sin, hadamard_q=hq, hadamard_k=hk, k_cache=k_cache,
+                               k_cache_scale=k_cache_scale, k_cache_index=idx.reshape(t), block_table=table)
 
 
 def config_lengths(cfg: int, seed: int = 0) -> List[int]:

@@ -29,7 +29,8 @@ def _declared():
 def test_header_symbols_are_exported(lib):
     names = _declared()
     assert {"pto_sfa_quant_launch", "pto_sfa_quant_workspace_bytes", "pto_li_decode_launch",
-            "pto_li_decode_workspace_bytes", "pto_last_error", "pto_version"} <= set(names)
+            "pto_li_decode_workspace_bytes", "pto_li_prolog_quant_launch", "pto_li_prolog_quant_workspace_bytes",
+            "pto_last_error", "pto_version"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
 
@@ -50,6 +51,14 @@ def test_pybind_workspace_and_argument_errors():
     assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 20, 0.04, 8) == 32 * 8 * 128 * (512 * 2 + 8)
     assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 0      # no split needed
     assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * 32768 * 4
+    # prolog: 4 int32 partial projections [t, 8192] + 112 block sums [t, 192] fp32
+    assert C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 64, 1 << 20) == 4 * 8 * 8192 * 4 + 112 * 8 * 192 * 4
+    with pytest.raises(ValueError):
+        C.li_prolog_quant_workspace_bytes(8, 7168, 1280, 64, 1 << 20)                # q_lora_rank not supported
+    with pytest.raises(ValueError):
+        C.li_prolog_quant_workspace_bytes(8, 7100, 1536, 64, 1 << 20)                # h not a multiple of 64
+    with pytest.raises(ValueError):
+        C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 65, 1 << 20)                # more than 64 heads
     with pytest.raises(ValueError):
         C.sfa_quant_workspace_bytes(1, 1, 128, 2, 2048, 128, 32, 4096, 0.04, 0)      # n_kv != 1
     with pytest.raises(ValueError):

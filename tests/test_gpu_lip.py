@@ -1,0 +1,101 @@
+"""Parity of the HIP lightning-indexer prolog (through the operator, pybind11 and the C ABI) against the
+CPU oracle.  The oracle fixes the order of every fp32 sum, so the bar is bit-exact: int8 query and key
+rows, fp16 scales, fp16 weights, and every byte of the key cache outside the scattered rows."""
+import numpy as np
+import pytest
+import torch
+
+import pypto_amd
+from oracle import lip_oracle as lo
+from pypto_amd.synthetic import gen_indexer_prolog_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def run_op(inp, separate_cache_out=False):
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    t = d.x.shape[0]
+    n = d.w_proj.shape[1]
+    q_int8 = torch.full([t, n, 128], -7, dtype=torch.int8, device=dev)
+    q_scale = torch.full([t, n, 1], -7, dtype=torch.float16, device=dev)
+    weights = torch.full([t, n], -7, dtype=torch.float16, device=dev)
+    if separate_cache_out:
+        k_out, ks_out = torch.zeros_like(d.k_cache), torch.zeros_like(d.k_cache_scale)
+    else:
+        k_out, ks_out = d.k_cache, d.k_cache_scale
+    ins = [pypto_amd.from_torch(v) for v in d.input_tensors()]
+    outs = [pypto_amd.from_torch(v) for v in (q_int8, q_scale, k_out, ks_out, weights)]
+    ret = pypto_amd.lightning_indexer_prolog_quant(*ins, *outs, pypto_amd.IndexerPrologQuantAttr(eps=1e-6),
+                                                   pypto_amd.IndexerPrologQuantConfigs())
+    assert ret is None
+    torch.cuda.synchronize()
+    return {"q_int8": q_int8.cpu().numpy(), "q_scale": q_scale.cpu().numpy()[..., 0], "k_cache": k_out.cpu().numpy(),
+            "k_cache_scale": ks_out.cpu().numpy(), "weights": weights.cpu().numpy()}
+
+
+def assert_exact(got, ref, what):
+    for name in ("q_int8", "q_scale", "weights", "k_cache", "k_cache_scale"):
+        g, r = got[name], ref[name]
+        assert g.shape == r.shape, (what, name, g.shape, r.shape)
+        gi, ri = g.view(np.uint8 if g.dtype == np.int8 else np.uint16), r.view(np.uint8 if r.dtype == np.int8 else np.uint16)
+        if not np.array_equal(gi, ri):
+            bad = np.argwhere(gi != ri)
+            first = tuple(bad[0])
+            raise AssertionError(f"{what}: {name}: {len(bad)} of {g.size} differ; first at {first}: got {g[first]} want {r[first]}")
+
+
+@pytest.mark.parametrize("b,s1,act,kw", [
+    (2, 2, [300, 129], dict(h=256, q_lora_rank=512, n_heads=4)),          # small everything
+    (1, 1, [77], dict(h=128, q_lora_rank=1024, n_heads=3)),               # one token, odd head count
+    (3, 1, [5, 128, 129], dict(h=512, q_lora_rank=1536, n_heads=8, affine_ln=True)),   # gamma/beta drawn at random
+    (5, 7, [900] * 5, dict(h=192, q_lora_rank=512, n_heads=2)),           # 35 tokens: two token blocks, ragged groups of 4
+])
+def test_prolog_small_shapes_bit_exact(b, s1, act, kw):
+    inp = gen_indexer_prolog_inputs(b, s1, act, seed=3 * b + s1, **kw)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert_exact(run_op(inp), ref, f"b={b} s1={s1} {kw}")
+
+
+def test_prolog_reference_case_b4_s1_2_s2_64k():
+    """Shapes of the reference's enabled test (deepseekv32_lightning_indexer_prolog_quant.py:431-446)."""
+    inp = gen_indexer_prolog_inputs(4, 2, [65536] * 4, seed=0)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    got = run_op(inp)
+    assert_exact(got, ref, "b4_s1_2_s2_64k")
+    # and the reference's own acceptance rule against the library-order evaluation of its golden
+    qi, qs, ki, ks, w = lo.indexer_prolog_library_order(*inp.input_tensors()[:13])
+    assert np.abs(got["q_int8"].astype(np.int32) - qi.numpy().astype(np.int32)).max() <= 1
+    assert (np.abs(got["q_scale"].astype(np.float32) - qs.float().numpy()) > 2.5e-5).mean() <= 0.005
+    assert np.abs(got["weights"].astype(np.float32) - w.float().numpy()).max() <= 2.5e-5
+    rows = inp.k_cache_index.numpy()
+    assert np.abs(got["k_cache"].reshape(-1, 128)[rows].astype(np.int32) - ki.numpy().astype(np.int32)).max() <= 1
+    assert np.abs(got["k_cache_scale"].reshape(-1)[rows].astype(np.float32) - ks.float().numpy()).max() <= 2.5e-5
+
+
+def test_prolog_separate_cache_output_and_skipped_indices():
+    inp = gen_indexer_prolog_inputs(2, 2, [300, 129], seed=5, h=256, q_lora_rank=512, n_heads=4)
+    inp.k_cache_index[1] = -1
+    inp.k_cache_index[2] = inp.k_cache.shape[0] * inp.k_cache.shape[1]
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert_exact(run_op(inp, separate_cache_out=True), ref, "separate outputs, two skipped indices")
+
+
+def test_prolog_zero_rows_and_repeatability():
+    """A token whose hidden state and query are zero: key path = layer norm of zeros (beta only), query rows
+    quantise to zeros with scale 0.  Two runs give identical bytes."""
+    inp = gen_indexer_prolog_inputs(1, 3, [400], seed=9, h=256, q_lora_rank=512, n_heads=4, affine_ln=True)
+    inp.x[1] = 0
+    inp.q_norm[1] = 0
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert not ref["q_int8"][1].any() and not ref["q_scale"][1].any()
+    a = run_op(inp)
+    assert_exact(a, ref, "zero token")
+    assert_exact(run_op(inp), a, "second run")
+
+
+def test_prolog_mtp_batch_t128():
+    """b=32, s1=4 (128 tokens: four token blocks) at the model's full projection sizes."""
+    inp = gen_indexer_prolog_inputs(32, 4, [2048 + 17 * i for i in range(32)], seed=2)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert_exact(run_op(inp), ref, "b32_s1_4")
