@@ -232,13 +232,14 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *args, void *hip_stream);
  *   weights        [t, n_heads]                  fp16   written
  *
  * Every fp32 sum has a fixed order, so results are reproducible bit for bit:
- * sums over h in blocks of 64 (ascending inside a block, blocks ascending), the
- * 128-term Hadamard sums ascending, the layer-norm means as balanced trees over
+ * sums over h in blocks of 64 (ascending inside a block), eight consecutive block
+ * sums added ascending into a group sum and the group sums added ascending; the
+ * 128-term Hadamard sums ascending; the layer-norm means as balanced trees over
  * neighbouring channels.  A row whose values are all zero quantises to zeros with
  * scale 0.  Cache indices outside [0, cache_rows) are skipped.
  *
  * Constraints: head_dim 128, rope 64, 1 <= n_heads <= 64, q_lora_rank in
- * {512, 1024, 1536}, h a positive multiple of 64, t >= 1.
+ * {512, 1024, 1536}, h a positive multiple of 64 up to 12288, t >= 1.
  */
 typedef struct PtoLiPrologQuantArgs {
     const void *x;

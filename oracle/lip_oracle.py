@@ -28,8 +28,9 @@ multiply-add and a multiply followed by an add give the same bits).
                         * f32(d**-0.5)))                                           (:272-275)
 
     blocked_dot   -- the reduction axis is cut into blocks of 64; a block is summed in
-                     ascending order starting from 0.0; block sums are added in ascending
-                     block order.
+                     ascending order starting from 0.0; eight consecutive block sums are added
+                     in ascending order (from 0.0) into a group sum; group sums are added in
+                     ascending order (from 0.0).
     pair_tree_sum -- 128 values: adjacent pairs are added, then adjacent pairs of those
                      sums, ... (a balanced binary tree over neighbours).
     quant_int8    -- amax = max|y|; s = rn32(127/amax); out = int8(rint(rn32(y*s)));
@@ -69,6 +70,7 @@ __all__ = [
 ]
 
 BLOCK_K = 64
+GROUP_BLOCKS = 8
 F32 = np.float32
 
 
@@ -86,7 +88,7 @@ def bf16_round(x: np.ndarray) -> np.ndarray:
     return u.astype(np.uint32).view(F32).reshape(x.shape)
 
 
-def blocked_dot(x: np.ndarray, w: np.ndarray, block: int = BLOCK_K) -> np.ndarray:
+def blocked_dot(x: np.ndarray, w: np.ndarray, block: int = BLOCK_K, group: int = GROUP_BLOCKS) -> np.ndarray:
     """[T,K] x [K,N] -> [T,N] fp32 in the fixed order stated in the module docstring."""
     x = np.asarray(x, F32)
     w = np.asarray(w, F32)
@@ -99,8 +101,11 @@ def blocked_dot(x: np.ndarray, w: np.ndarray, block: int = BLOCK_K) -> np.ndarra
     for i in range(block):
         part = part + xb[:, :, i, None] * wb[None, :, i, :]
     total = np.zeros((t, w.shape[1]), F32)
-    for c in range(nb):
-        total = total + part[:, c, :]
+    for g0 in range(0, nb, group):
+        gsum = np.zeros((t, w.shape[1]), F32)
+        for c in range(g0, min(g0 + group, nb)):
+            gsum = gsum + part[:, c, :]
+        total = total + gsum
     return total
 
 

@@ -201,8 +201,10 @@ int lip_check(const PtoLiPrologQuantArgs *a)
         return fail(PTO_E_INVALID_ARG, "li_prolog: n_heads must be in [1, %d] (got %lld)", pto::LIP_MAX_HEADS, (long long)a->n_heads);
     if (a->q_lora_rank != 512 && a->q_lora_rank != 1024 && a->q_lora_rank != 1536)
         return fail(PTO_E_INVALID_ARG, "li_prolog: q_lora_rank must be 512, 1024 or 1536 (got %lld)", (long long)a->q_lora_rank);
-    if (a->h < pto::LIP_XBLOCK || a->h % pto::LIP_XBLOCK != 0 || a->h > (1ll << 20))
-        return fail(PTO_E_INVALID_ARG, "li_prolog: h must be a positive multiple of %d (got %lld)", pto::LIP_XBLOCK, (long long)a->h);
+    const long long max_h = (long long)pto::LIP_MAX_XGROUPS * pto::LIP_XGROUP * pto::LIP_XBLOCK;
+    if (a->h < pto::LIP_XBLOCK || a->h % pto::LIP_XBLOCK != 0 || a->h > max_h)
+        return fail(PTO_E_INVALID_ARG, "li_prolog: h must be a positive multiple of %d, at most %lld (got %lld)", pto::LIP_XBLOCK,
+                    max_h, (long long)a->h);
     if (a->cache_rows < 1 || a->cache_rows > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "li_prolog: cache_rows out of range");
     if (!std::isfinite(a->eps) || a->eps < 0) return fail(PTO_E_INVALID_ARG, "li_prolog: eps must be finite and >= 0");
     return PTO_OK;

@@ -10,7 +10,8 @@
 //   weights bf16(x . w_proj) * n_heads^-1/2 * 128^-1/2 -> fp16
 // Every product of two bf16 values is exact in fp32, so each fp32 sum is fixed by its order alone.
 // The orders used here: sums over the hidden axis are cut into blocks of 64 (a block ascending from
-// 0.0, block sums added ascending); the Hadamard sums run over i ascending; the two layer-norm means
+// 0.0), eight consecutive block sums are added ascending into a group sum, group sums are added
+// ascending; the Hadamard sums run over i ascending; the two layer-norm means
 // are balanced binary trees over neighbouring channels.  No matrix-core instruction touches these
 // sums (its internal order is not specified); only the exact integer projection uses one.
 //
@@ -23,10 +24,10 @@
 //                       v_mfma_i32_32x32x32_i8 operands.  Partial int32 sums go to the workspace.
 //                       Hidden-axis jobs (block of 64 rows of wk and w_proj, 4 tokens): fp32 FMAs with
 //                       the hidden states as scalar operands; block sums go to the workspace.
-//   lip_finish_kernel   one wave per row.  Query rows: add the four partial sums, de-quantise, rope,
-//                       Hadamard (matrix staged in LDS once per workgroup), quantise, store.  Key
-//                       rows: add the block sums in order, layer norm, rope, Hadamard, quantise,
-//                       scatter.  Weight rows: add the block sums, scale, store.
+//   lip_finish_kernel   Query rows, one per wave: add the four partial sums, de-quantise, rope,
+//                       Hadamard (matrix staged in LDS once per workgroup), quantise, store.  Tokens,
+//                       one workgroup each: waves add the groups of block sums, then one wave finishes
+//                       the key row (layer norm, rope, Hadamard, quantise, scatter) and one the weights.
 #include "lip_kernels.h"
 #include "common.h"
 
@@ -285,27 +286,33 @@ __device__ __forceinline__ uint16_t quant_pair(const float y0, const float y1, u
     return 0;
 }
 
+constexpr int FIN_WAVES = 16;
+
 __device__ __forceinline__ void stage_matrix(uint32_t *dst, const uint16_t *src)
 {
     const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
     u32x4 *d = reinterpret_cast<u32x4 *>(dst);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d[i * 256 + threadIdx.x] = s[i * 256 + threadIdx.x];
+    for (int i = 0; i < 2; ++i) d[i * 1024 + threadIdx.x] = s[i * 1024 + threadIdx.x];
 }
 
-__global__ __launch_bounds__(256) void lip_finish_kernel(const LipParams p, const int q_wgs, const int k_wgs)
+// Workgroups [0, q_wgs): sixteen query rows (token, head) each, one per wave.
+// Workgroups [q_wgs, q_wgs + T): one token each -- waves add the groups of block sums over the hidden
+// axis (one group of eight blocks per wave and round), then wave 0 finishes the key row and wave 1 the
+// weights row.
+__global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
 {
     __shared__ __attribute__((aligned(16))) uint32_t hmat[LIP_DIM * 64];
-    __shared__ __attribute__((aligned(16))) float arow[4][LIP_DIM];
+    __shared__ __attribute__((aligned(16))) float arow[FIN_WAVES][LIP_DIM];
+    __shared__ __attribute__((aligned(16))) float gsum[LIP_MAX_XGROUPS][LIP_XCOLS];
     const int l = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ncols = p.n_heads * LIP_DIM;
-    const int nblk = p.h / LIP_XBLOCK;
-    int wg = blockIdx.x;
+    const int wg = blockIdx.x;
 
     if (wg < q_wgs) {
         stage_matrix(hmat, p.hq);
-        const int row = wg * 4 + w;                    // (token, head)
+        const int row = wg * FIN_WAVES + w;            // (token, head)
         const bool live = row < p.T * p.n_heads;
         const int t = live ? row / p.n_heads : 0;
         const int head = live ? row % p.n_heads : 0;
@@ -335,16 +342,41 @@ __global__ __launch_bounds__(256) void lip_finish_kernel(const LipParams p, cons
         }
         return;
     }
-    wg -= q_wgs;
-    if (wg < k_wgs) {
-        stage_matrix(hmat, p.hk);
-        const int tt = wg * 4 + w;
-        const bool live = tt < p.T;
-        const int t = live ? tt : 0;
+
+    const int t = wg - q_wgs;
+    const int nblk = p.h / LIP_XBLOCK;
+    const int ngroups = (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
+    stage_matrix(hmat, p.hk);
+    const bool pl = l < p.n_heads;
+    for (int g = w; g < ngroups; g += FIN_WAVES) {
+        const float *src = p.xpart + ((size_t)g * LIP_XGROUP * p.T + t) * LIP_XCOLS;
+        const int nb = nblk - g * LIP_XGROUP < LIP_XGROUP ? nblk - g * LIP_XGROUP : LIP_XGROUP;
+        f32x2 kv[LIP_XGROUP];
+        float wv[LIP_XGROUP];
+#pragma unroll
+        for (int i = 0; i < LIP_XGROUP; ++i) {
+            const float *r = src + (size_t)(i < nb ? i : 0) * p.T * LIP_XCOLS;
+            kv[i] = *reinterpret_cast<const f32x2 *>(r + 2 * l);
+            wv[i] = r[LIP_DIM + (pl ? l : 0)];
+        }
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < LIP_XGROUP; ++i) {
+            if (i < nb) {
+                s0 = __fadd_rn(s0, kv[i][0]);
+                s1 = __fadd_rn(s1, kv[i][1]);
+                s2 = __fadd_rn(s2, wv[i]);
+            }
+        }
+        f32x2 sv = {s0, s1};
+        *reinterpret_cast<f32x2 *>(&gsum[g][2 * l]) = sv;
+        gsum[g][LIP_DIM + l] = s2;
+    }
+    __syncthreads();
+    if (w == 0) {
         float v0 = 0.f, v1 = 0.f;
-        const float *src = p.xpart + (size_t)t * LIP_XCOLS + 2 * l;
-        for (int c = 0; c < nblk; ++c) {
-            const f32x2 v = *reinterpret_cast<const f32x2 *>(src + (size_t)c * p.T * LIP_XCOLS);
+        for (int g = 0; g < ngroups; ++g) {
+            const f32x2 v = *reinterpret_cast<const f32x2 *>(&gsum[g][2 * l]);
             v0 = __fadd_rn(v0, v[0]);
             v1 = __fadd_rn(v1, v[1]);
         }
@@ -359,31 +391,21 @@ __global__ __launch_bounds__(256) void lip_finish_kernel(const LipParams p, cons
         v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(g & 0xffff0000u)), __uint_as_float(b & 0xffff0000u)));
         rope_pair(v0, v1, p.cos, p.sin, t, l);
         f32x2 av = {v0, v1};
-        *reinterpret_cast<f32x2 *>(&arow[w][2 * l]) = av;
-        __syncthreads();
+        *reinterpret_cast<f32x2 *>(&arow[0][2 * l]) = av;
         float y0, y1;
-        hadamard_pair(arow[w], hmat, l, y0, y1);
+        hadamard_pair(arow[0], hmat, l, y0, y1);       // same wave wrote arow[0]: LDS operations of a wave stay in order
         uint16_t sc;
         const uint16_t q = quant_pair(y0, y1, sc);
-        if (live) {
-            const long long dst = p.k_cache_index[t];
-            if (dst >= 0 && dst < p.cache_rows) {
-                reinterpret_cast<uint16_t *>(p.k_cache + (size_t)dst * LIP_DIM)[l] = q;
-                if (l == 0) p.k_cache_scale[dst] = sc;
-            }
+        const long long dst = p.k_cache_index[t];
+        if (dst >= 0 && dst < p.cache_rows) {
+            reinterpret_cast<uint16_t *>(p.k_cache + (size_t)dst * LIP_DIM)[l] = q;
+            if (l == 0) p.k_cache_scale[dst] = sc;
         }
-        return;
-    }
-    wg -= k_wgs;
-    {
-        const int t = wg * 4 + w;
-        if (t < p.T && l < p.n_heads) {
-            float v = 0.f;
-            const float *src = p.xpart + (size_t)t * LIP_XCOLS + LIP_DIM + l;
-            for (int c = 0; c < nblk; ++c) v = __fadd_rn(v, src[(size_t)c * p.T * LIP_XCOLS]);
-            v = __fmul_rn(__fmul_rn(bf16_round_f32(v), p.w_mul0), p.w_mul1);
-            p.weights[(size_t)t * p.n_heads + l] = (uint16_t)(pack_f16x2(v, 0.f) & 0xffffu);
-        }
+    } else if (w == 1 && pl) {
+        float v = 0.f;
+        for (int g = 0; g < ngroups; ++g) v = __fadd_rn(v, gsum[g][LIP_DIM + l]);
+        v = __fmul_rn(__fmul_rn(bf16_round_f32(v), p.w_mul0), p.w_mul1);
+        p.weights[(size_t)t * p.n_heads + l] = (uint16_t)(pack_f16x2(v, 0.f) & 0xffffu);
     }
 }
 
@@ -405,9 +427,8 @@ hipError_t lip_launch(const LipParams &p, hipStream_t stream)
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const int q_wgs = (p.T * p.n_heads + 3) / 4;
-    const int k_wgs = (p.T + 3) / 4;
-    hipLaunchKernelGGL(lip_finish_kernel, dim3((unsigned)(q_wgs + 2 * k_wgs)), dim3(256), 0, stream, p, q_wgs, k_wgs);
+    const int q_wgs = (p.T * p.n_heads + FIN_WAVES - 1) / FIN_WAVES;
+    hipLaunchKernelGGL(lip_finish_kernel, dim3((unsigned)(q_wgs + p.T)), dim3(64 * FIN_WAVES), 0, stream, p, q_wgs);
     return hipGetLastError();
 }
 

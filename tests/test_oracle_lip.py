@@ -78,30 +78,43 @@ def test_q_linear_against_python_integers():
 
 def test_blocked_dot_order_exact_rational():
     rng = np.random.default_rng(2)
-    x = _bf16_vals(rng, (2, 128), 50.0)
-    w = _bf16_vals(rng, (128, 3), 50.0)
-    got = lo.blocked_dot(x, w, block=64)
+    x = _bf16_vals(rng, (2, 1152), 50.0)          # 18 blocks: groups of 8, 8 and 2
+    w = _bf16_vals(rng, (1152, 2), 50.0)
+    got = lo.blocked_dot(x, w)
     for t in range(2):
-        for n in range(3):
+        for n in range(2):
             total = 0.0
-            for c in range(2):
-                acc = 0.0
-                for k in range(64 * c, 64 * c + 64):
-                    acc = _rn32(Fraction(acc) + Fraction(float(x[t, k])) * Fraction(float(w[k, n])))
-                total = _rn32(Fraction(total) + Fraction(acc))
+            for g0 in range(0, 18, 8):
+                gsum = 0.0
+                for c in range(g0, min(g0 + 8, 18)):
+                    acc = 0.0
+                    for k in range(64 * c, 64 * c + 64):
+                        acc = _rn32(Fraction(acc) + Fraction(float(x[t, k])) * Fraction(float(w[k, n])))
+                    gsum = _rn32(Fraction(gsum) + Fraction(acc))
+                total = _rn32(Fraction(total) + Fraction(gsum))
             assert got[t, n] == np.float32(total)
 
 
 def test_blocked_dot_is_order_sensitive():
-    # 2**24 + 1 + 1 ... : the block structure decides whether the small terms survive
-    x = np.zeros((1, 128), np.float32)
-    w = np.ones((128, 1), np.float32)
+    # 2**24 followed by ones: where the ones meet the big term decides whether they survive
+    w = np.ones((1024, 1), np.float32)
+    x = np.zeros((1, 1024), np.float32)
     x[0, 0] = 2.0 ** 24
-    x[0, 64:] = 1.0
-    got = lo.blocked_dot(x, w, block=64)
-    # block 0 = 2**24, block 1 = 64 (exact), total = 2**24 + 64; a single ascending chain gives 2**24
-    assert got[0, 0] == np.float32(2.0 ** 24 + 64)
-    assert lo.blocked_dot(x, w, block=128)[0, 0] == np.float32(2.0 ** 24)
+    x[0, 64:128] = 1.0                             # block 1 of group 0
+    x[0, 512:] = 1.0                               # group 1
+    got = lo.blocked_dot(x, w)
+    # block level: 2**24 alone in block 0; block 1 = 64; group 0 = 2**24 + 64; group 1 = 512
+    assert got[0, 0] == np.float32(2.0 ** 24 + 64 + 512)
+    # a single ascending chain loses every one of them
+    assert lo.blocked_dot(x, w, block=1024)[0, 0] == np.float32(2.0 ** 24)
+    # the second level matters too: 2**24 in block 0, every later block sums to exactly 1.0.  With groups
+    # of eight the seven ones of group 0 are lost one by one but group 1 arrives as 8.0 and survives;
+    # one chain over all sixteen block sums loses all fifteen.
+    x2 = np.full((1, 1024), 1.0 / 64, np.float32)
+    x2[0, :64] = 0.0
+    x2[0, 0] = 2.0 ** 24
+    assert lo.blocked_dot(x2, w)[0, 0] == np.float32(2.0 ** 24 + 8)
+    assert lo.blocked_dot(x2, w, group=16)[0, 0] == np.float32(2.0 ** 24)
 
 
 def test_pair_tree_sum_order():
