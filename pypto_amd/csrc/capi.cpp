@@ -361,7 +361,7 @@ int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
     if (!a->workspace || a->workspace_bytes < need)
         return fail(PTO_E_WORKSPACE, "li_prolog: workspace of %zu bytes required, %zu given", need,
                     a->workspace ? a->workspace_bytes : (size_t)0);
-    const void *aligned[] = {a->x, a->q_norm, a->q_norm_scale, a->w_qb, a->w_qb_scale, a->wk, a->ln_gamma_k, a->ln_beta_k,
+    const void *aligned[] = {a->x, a->q_norm, a->q_norm_scale, a->w_qb, a->w_qb_scale, a->wk, a->w_proj, a->ln_gamma_k, a->ln_beta_k,
                              a->cos_idx_rope, a->sin_idx_rope, a->hadamard_q, a->hadamard_k, a->k_cache, a->q_int8, a->workspace};
     for (const void *ptr : aligned)
         if (reinterpret_cast<uintptr_t>(ptr) & 15)

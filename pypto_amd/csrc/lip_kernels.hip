@@ -16,14 +16,15 @@
 // sums (its internal order is not specified); only the exact integer projection uses one.
 //
 // Two launches:
-//   lip_linear_kernel   one wave per job.  Query jobs (head, quarter of the reduction axis, block of
-//                       32 tokens): the quarter tile of w_qb (q_lora/4 rows x 128 bytes) and the
-//                       token rows travel to LDS by LDS-DMA, all requests issued up front; each
-//                       32-row step is consumed as soon as its requests have landed (they complete in
-//                       order): 4x4 byte transposes (v_perm_b32) turn the row-major tile into
-//                       v_mfma_i32_32x32x32_i8 operands.  Partial int32 sums go to the workspace.
-//                       Hidden-axis jobs (block of 64 rows of wk and w_proj, 4 tokens): fp32 FMAs with
-//                       the hidden states as scalar operands; block sums go to the workspace.
+//   lip_linear_kernel   workgroups of four independent waves.  Two of them share a query job (head,
+//                       quarter of the reduction axis, block of 32 tokens), one half each: the tile of
+//                       w_qb (rows x 128 bytes) and the token rows travel to LDS by LDS-DMA, all
+//                       requests issued up front; 32-row steps are consumed as their requests land
+//                       (they complete in order): 4x4 byte transposes (v_perm_b32) turn the row-major
+//                       tile into v_mfma_i32_32x32x32_i8 operands.  The two halves are added through
+//                       LDS and the partial int32 sums go to the workspace.  The other two waves take
+//                       hidden-axis jobs (block of 64 rows of wk or of w_proj, 4 tokens): fp32 FMAs
+//                       with the hidden states as scalar operands; block sums go to the workspace.
 //   lip_finish_kernel   Query rows, one per wave: add the four partial sums, de-quantise, rope,
 //                       Hadamard (matrix staged in LDS once per workgroup), quantise, store.  Tokens,
 //                       one workgroup each: waves add the groups of block sums, then one wave finishes
@@ -77,53 +78,51 @@ __device__ __forceinline__ float bf16_round_f32(const float v)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Query projection job.  STEPS = q_lora / 4 / 32 steps of 32 reduction rows.
-// LDS: [tile: 32*STEPS rows x 128 bytes][token operands: STEPS x 1024 bytes].
+// Query projection: one workgroup per (head, quarter of the reduction axis, block of 32 tokens); its
+// waves 0 and 1 take one half of the quarter each (HS steps of 32 rows).
+// LDS region of a wave: [tile: 32*HS rows x 128 bytes][token operands: HS x 1024 bytes].
 // Matrix product per step: A = 32 output columns x 32 rows of the tile (lane (j, g) holds rows
 // 16g..16g+15 of column 4j+i for product i), B = 32 tokens x the same 32 rows of q_norm, so that
 // accumulator register r of lane l holds column 4*(8*(r/4) + 4*(l/32) + r%4) + i, token l%32.
-template <int STEPS>
-__device__ __forceinline__ void q_linear_job(const LipParams &p, uint8_t *smem, const int job)
+template <int HS>
+__device__ __forceinline__ void q_half_job(const LipParams &p, uint8_t *region, const int job, const int half, i32x16 (&acc)[4])
 {
-    const int l = threadIdx.x;
+    const int l = threadIdx.x & 63;
     const int ncols = p.n_heads * LIP_DIM;
     const int kq = job & (LIP_KSPLIT - 1);
     const int head = (job >> 2) % p.n_heads;
     const int tb = (job >> 2) / p.n_heads;
-    constexpr int KPER = STEPS * 32;
-    constexpr int NW = KPER / 8;                       // tile requests of 8 rows each
-    const uint32_t tile = (uint32_t)(uintptr_t)(lds_byte_t *)smem;
-    const uint32_t tok = tile + KPER * 128;
+    constexpr int KH = HS * 32;                        // rows of this wave
+    constexpr int NW = KH / 8;                         // tile requests of 8 rows each
+    const int k0 = (kq * 2 + half) * KH;
+    const uint32_t tile = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+    const uint32_t tok = tile + KH * 128;
 
-    // token operands first (they complete first), then the tile
+    // token operands and the tile: every request is issued before the first wait.  The loops stay
+    // rolled: straight-line code that runs once is bound by instruction fetch.
     {
         int t = tb * 32 + (l & 31);
         t = t < p.T ? t : p.T - 1;
-        const int8_t *src = p.q_norm + (size_t)t * p.q_lora + kq * KPER + 16 * (l >> 5);
-#pragma unroll
-        for (int s = 0; s < STEPS; ++s) dma16(src + 32 * s, tok + 1024 * s);
+        const int8_t *src = p.q_norm + (size_t)t * p.q_lora + k0 + 16 * (l >> 5);
+#pragma unroll 1
+        for (int s = 0; s < HS; ++s) dma16(src + 32 * s, tok + 1024 * s);
     }
     {
-        const int8_t *src = p.w_qb + ((size_t)kq * KPER + (l >> 3)) * ncols + head * LIP_DIM + 16 * (l & 7);
-#pragma unroll
+        const int8_t *src = p.w_qb + ((size_t)k0 + (l >> 3)) * ncols + head * LIP_DIM + 16 * (l & 7);
+#pragma unroll 2
         for (int i = 0; i < NW; ++i) dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
     }
-
-    i32x16 acc[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
-
-    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(smem);
+    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(region);
     const int rd = (16 * (l >> 5)) * 32 + (l & 31);     // dword index of this lane's first row of a step
+    // The tile arrives at the pace of the memory system; each step starts as soon as its four
+    // requests have landed (requests complete in order), so only the last step trails the arrival.
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
+    for (int s = 0; s < HS; ++s) {
         wait_vm_le(NW - 4 * (s + 1));
         uint32_t d[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
-        const i32x4 b = *reinterpret_cast<const i32x4 *>(smem + KPER * 128 + 1024 * s + 16 * l);
+        const i32x4 b = *reinterpret_cast<const i32x4 *>(region + KH * 128 + 1024 * s + 16 * l);
         i32x4 a[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -137,91 +136,207 @@ __device__ __forceinline__ void q_linear_job(const LipParams &p, uint8_t *smem, 
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
     }
-
-    const int t = tb * 32 + (l & 31);
-    if (t < p.T) {
-        int32_t *dst = p.qpart + ((size_t)kq * p.T + t) * ncols + head * LIP_DIM;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
-            i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-            *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
-        }
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
-// Hidden-axis job: block c of 64 rows of wk (lane l: columns 2l, 2l+1) and w_proj (lane l: column l),
-// tokens t0..t0+3.  The hidden states are wave-uniform and are read through the scalar path.
-__device__ __forceinline__ void x_linear_job(const LipParams &p, const int job)
+// Hidden-axis jobs: block c of 64 rows, tokens t0, t0+1.  Even jobs take wk (lane l: columns 2l,
+// 2l+1), odd jobs w_proj (lane l: column l).  The block of weights (contiguous in memory) travels to
+// the wave's LDS region by LDS-DMA, the two token slices are converted to fp32 on the way in; the
+// product loop reads weights per lane and the hidden states as broadcasts.
+constexpr int XW_BYTES = LIP_XBLOCK * LIP_DIM * 2;     // 16 KiB: a block of wk
+constexpr int XTOK = 2;                               // tokens per hidden-axis job
+constexpr int X_REGION_BYTES = XW_BYTES + XTOK * LIP_XBLOCK * 4;
+constexpr int LIN_XWAVES = 4;
+
+__device__ __forceinline__ void x_linear_job(const LipParams &p, uint8_t *region, const int job)
 {
-    const int l = threadIdx.x;
+    const int l = threadIdx.x & 63;
     const int nblk = p.h / LIP_XBLOCK;
-    const int c = job % nblk;
-    const int t0 = (job / nblk) * 4;
+    const int c = (job >> 1) % nblk;
+    const int t0 = ((job >> 1) / nblk) * XTOK;
     const int k0 = c * LIP_XBLOCK;
-    const uint32_t *wk32 = reinterpret_cast<const uint32_t *>(p.wk) + (size_t)k0 * 64 + l;
-    const bool pl = l < p.n_heads;
-    const uint16_t *wp = p.w_proj + (size_t)k0 * p.n_heads + (pl ? l : 0);
-    const uint32_t *xr[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const int tt = t0 + t < p.T ? t0 + t : p.T - 1;
-        xr[t] = reinterpret_cast<const uint32_t *>(p.x + (size_t)tt * p.h + k0);
+    const bool proj = job & 1;
+    const uint32_t wdst = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+    float *xs = reinterpret_cast<float *>(region + XW_BYTES);          // [XTOK][64]
+
+    // the block: rows k0..k0+63 of wk (256 bytes each) or of w_proj (2*n_heads bytes each), contiguous
+    const int bytes = proj ? LIP_XBLOCK * p.n_heads * 2 : XW_BYTES;
+    const uint8_t *wsrc = proj ? reinterpret_cast<const uint8_t *>(p.w_proj) + (size_t)k0 * p.n_heads * 2
+                               : reinterpret_cast<const uint8_t *>(p.wk) + (size_t)k0 * LIP_DIM * 2;
+#pragma unroll 1
+    for (int off = 0; off < bytes; off += 1024) {
+        int o = off + 16 * l;
+        o = o < bytes - 16 ? o : bytes - 16;            // lanes past the end re-read its last 16 bytes
+        dma16(wsrc + o, wdst + off);
     }
-    // the whole block of weights is requested before the first use
-    uint32_t wv[LIP_XBLOCK];
-    uint16_t pv[LIP_XBLOCK];
-#pragma unroll
-    for (int kk = 0; kk < LIP_XBLOCK; ++kk) wv[kk] = wk32[(size_t)kk * 64];
-#pragma unroll
-    for (int kk = 0; kk < LIP_XBLOCK; ++kk) pv[kk] = wp[(size_t)kk * p.n_heads];
-    float a0[4] = {0.f, 0.f, 0.f, 0.f}, a1[4] = {0.f, 0.f, 0.f, 0.f}, a2[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < LIP_XBLOCK; kk += 2) {
-        const float wa0 = __uint_as_float(wv[kk] << 16), wa1 = __uint_as_float(wv[kk] & 0xffff0000u);
-        const float wb0 = __uint_as_float(wv[kk + 1] << 16), wb1 = __uint_as_float(wv[kk + 1] & 0xffff0000u);
-        const float pa = bf16_bits_to_f32(pv[kk]);
-        const float pb = bf16_bits_to_f32(pv[kk + 1]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const uint32_t xv = xr[t][kk >> 1];
-            const float xa = __uint_as_float(xv << 16), xb = __uint_as_float(xv & 0xffff0000u);
-            a0[t] = __builtin_fmaf(xa, wa0, a0[t]);
-            a1[t] = __builtin_fmaf(xa, wa1, a1[t]);
-            a2[t] = __builtin_fmaf(xa, pa, a2[t]);
-            a0[t] = __builtin_fmaf(xb, wb0, a0[t]);
-            a1[t] = __builtin_fmaf(xb, wb1, a1[t]);
-            a2[t] = __builtin_fmaf(xb, pb, a2[t]);
-        }
+    {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + l/32
+        const int t = t0 + (l >> 5);
+        const int tt = t < p.T ? t : p.T - 1;
+        const uint32_t xv = reinterpret_cast<const uint32_t *>(p.x + (size_t)tt * p.h + k0)[l & 31];
+        f32x2 v = {__uint_as_float(xv << 16), __uint_as_float(xv & 0xffff0000u)};
+        *reinterpret_cast<f32x2 *>(xs + (l >> 5) * LIP_XBLOCK + 2 * (l & 31)) = v;
     }
+    VM_WAIT(0);
+    // the wave reads back only what it wrote or requested itself: no barrier
+
+    if (!proj) {
+        const uint32_t *wl = reinterpret_cast<const uint32_t *>(region) + l;
+        float a0[XTOK] = {0.f, 0.f}, a1[XTOK] = {0.f, 0.f};
+#pragma unroll 2
+        for (int kk = 0; kk < LIP_XBLOCK; kk += 4) {
+            f32x4 xv[XTOK];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        if (t0 + t < p.T) {
-            float *dst = p.xpart + ((size_t)c * p.T + t0 + t) * LIP_XCOLS;
-            f32x2 v = {a0[t], a1[t]};
-            *reinterpret_cast<f32x2 *>(dst + 2 * l) = v;
-            if (pl) dst[LIP_DIM + l] = a2[t];
+            for (int t = 0; t < XTOK; ++t) xv[t] = *reinterpret_cast<const f32x4 *>(xs + t * LIP_XBLOCK + kk);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t wv = wl[(kk + j) * 64];
+                const float w0 = __uint_as_float(wv << 16), w1 = __uint_as_float(wv & 0xffff0000u);
+#pragma unroll
+                for (int t = 0; t < XTOK; ++t) {
+                    a0[t] = __builtin_fmaf(xv[t][j], w0, a0[t]);
+                    a1[t] = __builtin_fmaf(xv[t][j], w1, a1[t]);
+                }
+            }
         }
+#pragma unroll
+        for (int t = 0; t < XTOK; ++t) {
+            if (t0 + t < p.T) {
+                f32x2 v = {a0[t], a1[t]};
+                *reinterpret_cast<f32x2 *>(p.xpart + ((size_t)c * p.T + t0 + t) * LIP_XCOLS + 2 * l) = v;
+            }
+        }
+    } else {
+        const bool pl = l < p.n_heads;
+        const uint16_t *wl = reinterpret_cast<const uint16_t *>(region) + (pl ? l : 0);
+        float a2[XTOK] = {0.f, 0.f};
+#pragma unroll 2
+        for (int kk = 0; kk < LIP_XBLOCK; kk += 4) {
+            f32x4 xv[XTOK];
+#pragma unroll
+            for (int t = 0; t < XTOK; ++t) xv[t] = *reinterpret_cast<const f32x4 *>(xs + t * LIP_XBLOCK + kk);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float w2 = bf16_bits_to_f32(wl[(kk + j) * p.n_heads]);
+#pragma unroll
+                for (int t = 0; t < XTOK; ++t) a2[t] = __builtin_fmaf(xv[t][j], w2, a2[t]);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < XTOK; ++t)
+            if (t0 + t < p.T && pl) p.xpart[((size_t)c * p.T + t0 + t) * LIP_XCOLS + LIP_DIM + l] = a2[t];
     }
 }
 
-template <int STEPS>
-__global__ __launch_bounds__(64) void lip_linear_kernel(const LipParams p, const int q_jobs)
+constexpr int LIN_RED_BYTES = 16 * 64 * 16;           // one wave's accumulators, 16 bytes per (register, lane)
+
+template <int HS>
+constexpr int lin_region_bytes()
 {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lip_smem[];
+    return HS * (32 * 128 + 1024) > LIN_RED_BYTES ? HS * (32 * 128 + 1024) : LIN_RED_BYTES;
+}
+template <int HS>
+constexpr int lin_lds_bytes()
+{
+    return 2 * lin_region_bytes<HS>() + LIN_XWAVES * X_REGION_BYTES;
+}
+
+// Workgroup of six waves, no dependencies among them except the final pairwise sum of the two query
+// waves: waves 0 and 1 run the two halves of query job blockIdx.x, waves 2..5 walk the hidden-axis jobs.
+template <int HS>
+__global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const LipParams p, const int q_jobs, const int x_jobs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lip_smem[lin_lds_bytes<HS>()];
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l = threadIdx.x & 63;
     const int job = blockIdx.x;
-    if (job < q_jobs) q_linear_job<STEPS>(p, lip_smem, job);
-    else x_linear_job(p, job - q_jobs);
+    const bool qwave = w < 2 && job < q_jobs;
+    uint8_t *region = lip_smem + (w & 1) * lin_region_bytes<HS>();
+    i32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+
+    if (qwave) {
+        q_half_job<HS>(p, region, job, w, acc);
+        if (w == 1) {
+            i32x4 *red = reinterpret_cast<i32x4 *>(region);       // its own tile is consumed
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+                red[r * 64 + l] = v;
+            }
+        }
+    } else if (w >= 2) {
+        uint8_t *xregion = lip_smem + 2 * lin_region_bytes<HS>() + (w - 2) * X_REGION_BYTES;
+        for (int j = job * LIN_XWAVES + (w - 2); j < x_jobs; j += gridDim.x * LIN_XWAVES) x_linear_job(p, xregion, j);
+    }
+    __syncthreads();
+    if (qwave && w == 0) {
+        const i32x4 *red = reinterpret_cast<const i32x4 *>(lip_smem + lin_region_bytes<HS>());
+        const int ncols = p.n_heads * LIP_DIM;
+        const int kq = job & (LIP_KSPLIT - 1);
+        const int head = (job >> 2) % p.n_heads;
+        const int t = ((job >> 2) / p.n_heads) * 32 + (l & 31);
+        if (t < p.T) {
+            int32_t *dst = p.qpart + ((size_t)kq * p.T + t) * ncols + head * LIP_DIM;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
+                const i32x4 o = red[r * 64 + l];
+                i32x4 v = {acc[0][r] + o[0], acc[1][r] + o[1], acc[2][r] + o[2], acc[3][r] + o[3]};
+                *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
+            }
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
 // Second launch.
 
+// Cross-lane exchanges without LDS traffic.  dpp_f32 reads another lane of the same row of 16;
+// row_swap16 / half_swap32 return {own-side, other-side} copies across rows of 16 / halves of 32
+// (v_permlane16_swap, v_permlane32_swap with both operands equal).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(const float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int DPP_XOR1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141;  // lane i of a group of 8 reads lane 7-i
+constexpr int DPP_MIRROR = 0x140;     // lane i of a row of 16 reads lane 15-i
+
+// value held by lane l ^ 16
+__device__ __forceinline__ float xor16_f32(const float v, const int l)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    // r[0]: rows 0,0,2,2 of v;  r[1]: rows 1,1,3,3
+    return __uint_as_float((l & 16) ? r[0] : r[1]);
+}
+
+// combine(own, partner) over the whole wave where combine is commutative and every step leaves all
+// lanes of the finished group with the same bits: xor 1, xor 2, then mirrors within 8 and 16 lanes
+// (the mirrored lane lies in the other half, which is uniform), then the row and half swaps.
+#define WAVE_BUTTERFLY(v, OP)                                                                              \
+    do {                                                                                                   \
+        v = OP(v, dpp_f32<DPP_XOR1>(v));                                                                   \
+        v = OP(v, dpp_f32<DPP_XOR2>(v));                                                                   \
+        v = OP(v, dpp_f32<DPP_HALF_MIRROR>(v));                                                            \
+        v = OP(v, dpp_f32<DPP_MIRROR>(v));                                                                 \
+        {                                                                                                  \
+            const auto r_ = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false); \
+            v = OP(__uint_as_float(r_[0]), __uint_as_float(r_[1]));                                        \
+        }                                                                                                  \
+        {                                                                                                  \
+            const auto r_ = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false); \
+            v = OP(__uint_as_float(r_[0]), __uint_as_float(r_[1]));                                        \
+        }                                                                                                  \
+    } while (0)
+
 __device__ __forceinline__ float wave_max_f32(float v)
 {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
+    WAVE_BUTTERFLY(v, fmaxf);
     return v;
 }
 
@@ -229,20 +344,17 @@ __device__ __forceinline__ float wave_max_f32(float v)
 __device__ __forceinline__ float pair_tree_sum(const float v0, const float v1)
 {
     float s = __fadd_rn(v0, v1);
-#pragma unroll
-    for (int m = 1; m <= 32; m <<= 1) s = __fadd_rn(s, __shfl_xor(s, m));
+    WAVE_BUTTERFLY(s, __fadd_rn);
     return s;
 }
 
 // rope on channels 0..63 (lanes 0..31 hold channels 2l, 2l+1); the rotation partner of channel i is
 // i+32 (negated) for i < 32 and i-32 otherwise: lane l ^ 16.  Results rounded to bf16.
-__device__ __forceinline__ void rope_pair(float &v0, float &v1, const uint16_t *cos, const uint16_t *sin, const int t, const int l)
+__device__ __forceinline__ void rope_pair(float &v0, float &v1, const uint32_t c, const uint32_t s, const int l)
 {
-    const float p0 = __shfl_xor(v0, 16);
-    const float p1 = __shfl_xor(v1, 16);
+    const float p0 = xor16_f32(v0, l);
+    const float p1 = xor16_f32(v1, l);
     if (l < 32) {
-        const uint32_t c = reinterpret_cast<const uint32_t *>(cos + (size_t)t * LIP_ROPE)[l];
-        const uint32_t s = reinterpret_cast<const uint32_t *>(sin + (size_t)t * LIP_ROPE)[l];
         const float sg = l < 16 ? -1.0f : 1.0f;
         // both products are exact, so the fused form rounds once, like product + product
         const float r0 = __builtin_fmaf(v0, __uint_as_float(c << 16), (sg * p0) * __uint_as_float(s << 16));
@@ -251,21 +363,45 @@ __device__ __forceinline__ void rope_pair(float &v0, float &v1, const uint16_t *
         v1 = bf16_round_f32(r1);
     }
 }
+// the cos / sin pair of lane l (channels 2l, 2l+1 of token t); lanes 32..63 read lane l-32's, unused
+__device__ __forceinline__ uint32_t rope_coef(const uint16_t *tab, const int t, const int l)
+{
+    return reinterpret_cast<const uint32_t *>(tab + (size_t)t * LIP_ROPE)[l & 31];
+}
 
 // y[j] = sum_i a[i] * H[i][j], i ascending; lane l computes columns 2l and 2l+1.  a: this wave's 128
-// floats in LDS, hmat: the matrix in LDS as stored (row-major bf16).
-__device__ __forceinline__ void hadamard_pair(const float *a, const uint32_t *hmat, const int l, float &y0, float &y1)
+// floats in LDS, hmat: the matrix in LDS as fp32, row-major.  Chunks of 16 rows are read one chunk
+// ahead of the multiply-adds that consume them.
+struct HadChunk {
+    f32x4 a[4];
+    f32x2 h[16];
+};
+__device__ __forceinline__ void had_load(HadChunk &c, const float *a, const float *hmat, const int l, const int i0)
+{
+#pragma unroll
+    for (int u = 0; u < 4; ++u) c.a[u] = *reinterpret_cast<const f32x4 *>(a + i0 + 4 * u);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) c.h[u] = *reinterpret_cast<const f32x2 *>(hmat + (i0 + u) * LIP_DIM + 2 * l);
+}
+__device__ __forceinline__ void had_fma(const HadChunk &c, float &o0, float &o1)
+{
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        o0 = __builtin_fmaf(c.a[u >> 2][u & 3], c.h[u][0], o0);
+        o1 = __builtin_fmaf(c.a[u >> 2][u & 3], c.h[u][1], o1);
+    }
+}
+__device__ __forceinline__ void hadamard_pair(const float *a, const float *hmat, const int l, float &y0, float &y1)
 {
     float o0 = 0.f, o1 = 0.f;
-#pragma unroll 4
-    for (int i = 0; i < LIP_DIM; i += 4) {
-        const f32x4 av = *reinterpret_cast<const f32x4 *>(a + i);
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint32_t hv = hmat[(i + u) * 64 + l];
-            o0 = __builtin_fmaf(av[u], __uint_as_float(hv << 16), o0);
-            o1 = __builtin_fmaf(av[u], __uint_as_float(hv & 0xffff0000u), o1);
-        }
+    HadChunk c0, c1;
+    had_load(c0, a, hmat, l, 0);
+#pragma unroll 1
+    for (int i = 0; i < LIP_DIM; i += 32) {
+        had_load(c1, a, hmat, l, i + 16);
+        had_fma(c0, o0, o1);
+        had_load(c0, a, hmat, l, i + 32 < LIP_DIM ? i + 32 : 0);
+        had_fma(c1, o0, o1);
     }
     y0 = bf16_round_f32(o0);
     y1 = bf16_round_f32(o1);
@@ -286,23 +422,33 @@ __device__ __forceinline__ uint16_t quant_pair(const float y0, const float y1, u
     return 0;
 }
 
-constexpr int FIN_WAVES = 16;
+constexpr int FIN_WAVES = 8;
 
-__device__ __forceinline__ void stage_matrix(uint32_t *dst, const uint16_t *src)
+// the 128x128 bf16 matrix, widened to fp32, into LDS
+__device__ __forceinline__ void stage_matrix(float *dst, const uint16_t *src)
 {
     const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
-    u32x4 *d = reinterpret_cast<u32x4 *>(dst);
+    constexpr int NT = 64 * FIN_WAVES;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) d[i * 1024 + threadIdx.x] = s[i * 1024 + threadIdx.x];
+    for (int i = 0; i < 2048 / NT; ++i) {
+        const u32x4 v = s[i * NT + threadIdx.x];
+        f32x4 lo = {__uint_as_float(v[0] << 16), __uint_as_float(v[0] & 0xffff0000u), __uint_as_float(v[1] << 16),
+                    __uint_as_float(v[1] & 0xffff0000u)};
+        f32x4 hi = {__uint_as_float(v[2] << 16), __uint_as_float(v[2] & 0xffff0000u), __uint_as_float(v[3] << 16),
+                    __uint_as_float(v[3] & 0xffff0000u)};
+        f32x4 *d = reinterpret_cast<f32x4 *>(dst + (size_t)(i * NT + threadIdx.x) * 8);
+        d[0] = lo;
+        d[1] = hi;
+    }
 }
 
-// Workgroups [0, q_wgs): sixteen query rows (token, head) each, one per wave.
+// Workgroups [0, q_wgs): FIN_WAVES query rows (token, head) each, one per wave.
 // Workgroups [q_wgs, q_wgs + T): one token each -- waves add the groups of block sums over the hidden
-// axis (one group of eight blocks per wave and round), then wave 0 finishes the key row and wave 1 the
+// axis (two groups of eight blocks per wave and round), then wave 0 finishes the key row and wave 1 the
 // weights row.
 __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
 {
-    __shared__ __attribute__((aligned(16))) uint32_t hmat[LIP_DIM * 64];
+    __shared__ __attribute__((aligned(16))) float hmat[LIP_DIM * LIP_DIM];
     __shared__ __attribute__((aligned(16))) float arow[FIN_WAVES][LIP_DIM];
     __shared__ __attribute__((aligned(16))) float gsum[LIP_MAX_XGROUPS][LIP_XCOLS];
     const int l = threadIdx.x & 63;
@@ -326,9 +472,10 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipPar
         }
         const float ts = p.q_norm_scale[t];
         const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
+        const uint32_t rc = rope_coef(p.cos, t, l), rs = rope_coef(p.sin, t, l);
         float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
         float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
-        rope_pair(v0, v1, p.cos, p.sin, t, l);
+        rope_pair(v0, v1, rc, rs, l);
         f32x2 av = {v0, v1};
         *reinterpret_cast<f32x2 *>(&arow[w][2 * l]) = av;
         __syncthreads();
@@ -348,29 +495,45 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipPar
     const int ngroups = (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
     stage_matrix(hmat, p.hk);
     const bool pl = l < p.n_heads;
-    for (int g = w; g < ngroups; g += FIN_WAVES) {
-        const float *src = p.xpart + ((size_t)g * LIP_XGROUP * p.T + t) * LIP_XCOLS;
-        const int nb = nblk - g * LIP_XGROUP < LIP_XGROUP ? nblk - g * LIP_XGROUP : LIP_XGROUP;
-        f32x2 kv[LIP_XGROUP];
-        float wv[LIP_XGROUP];
+    // everything wave 0 needs later is requested now
+    const uint32_t rc = rope_coef(p.cos, t, l), rs = rope_coef(p.sin, t, l);
+    const uint32_t gm = reinterpret_cast<const uint32_t *>(p.gamma)[l];
+    const uint32_t bt = reinterpret_cast<const uint32_t *>(p.beta)[l];
+    const long long dst = p.k_cache_index[t];
+    for (int g0 = w; g0 < ngroups; g0 += 2 * FIN_WAVES) {
+        f32x2 kv[2][LIP_XGROUP];
+        float wv[2][LIP_XGROUP];
+        int nb[2];
 #pragma unroll
-        for (int i = 0; i < LIP_XGROUP; ++i) {
-            const float *r = src + (size_t)(i < nb ? i : 0) * p.T * LIP_XCOLS;
-            kv[i] = *reinterpret_cast<const f32x2 *>(r + 2 * l);
-            wv[i] = r[LIP_DIM + (pl ? l : 0)];
-        }
-        float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+        for (int u = 0; u < 2; ++u) {
+            const int g = g0 + u * FIN_WAVES;
+            const int left = nblk - g * LIP_XGROUP;
+            nb[u] = left < 0 ? 0 : (left < LIP_XGROUP ? left : LIP_XGROUP);
+            const float *src = p.xpart + ((size_t)(nb[u] ? g : 0) * LIP_XGROUP * p.T + t) * LIP_XCOLS;
 #pragma unroll
-        for (int i = 0; i < LIP_XGROUP; ++i) {
-            if (i < nb) {
-                s0 = __fadd_rn(s0, kv[i][0]);
-                s1 = __fadd_rn(s1, kv[i][1]);
-                s2 = __fadd_rn(s2, wv[i]);
+            for (int i = 0; i < LIP_XGROUP; ++i) {
+                const float *r = src + (size_t)(i < nb[u] ? i : 0) * p.T * LIP_XCOLS;
+                kv[u][i] = *reinterpret_cast<const f32x2 *>(r + 2 * l);
+                wv[u][i] = r[LIP_DIM + (pl ? l : 0)];
             }
         }
-        f32x2 sv = {s0, s1};
-        *reinterpret_cast<f32x2 *>(&gsum[g][2 * l]) = sv;
-        gsum[g][LIP_DIM + l] = s2;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            if (nb[u] == 0) continue;
+            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < LIP_XGROUP; ++i) {
+                if (i < nb[u]) {
+                    s0 = __fadd_rn(s0, kv[u][i][0]);
+                    s1 = __fadd_rn(s1, kv[u][i][1]);
+                    s2 = __fadd_rn(s2, wv[u][i]);
+                }
+            }
+            const int g = g0 + u * FIN_WAVES;
+            f32x2 sv = {s0, s1};
+            *reinterpret_cast<f32x2 *>(&gsum[g][2 * l]) = sv;
+            gsum[g][LIP_DIM + l] = s2;
+        }
     }
     __syncthreads();
     if (w == 0) {
@@ -385,18 +548,15 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipPar
         const float d0 = __fsub_rn(v0, mean), d1 = __fsub_rn(v1, mean);
         const float var = __fmul_rn(pair_tree_sum(__fmul_rn(d0, d0), __fmul_rn(d1, d1)), 1.0f / LIP_DIM);
         const float sd = __fsqrt_rn(__fadd_rn(var, p.eps));
-        const uint32_t g = reinterpret_cast<const uint32_t *>(p.gamma)[l];
-        const uint32_t b = reinterpret_cast<const uint32_t *>(p.beta)[l];
-        v0 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d0, sd), __uint_as_float(g << 16)), __uint_as_float(b << 16)));
-        v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(g & 0xffff0000u)), __uint_as_float(b & 0xffff0000u)));
-        rope_pair(v0, v1, p.cos, p.sin, t, l);
+        v0 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d0, sd), __uint_as_float(gm << 16)), __uint_as_float(bt << 16)));
+        v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(gm & 0xffff0000u)), __uint_as_float(bt & 0xffff0000u)));
+        rope_pair(v0, v1, rc, rs, l);
         f32x2 av = {v0, v1};
         *reinterpret_cast<f32x2 *>(&arow[0][2 * l]) = av;
         float y0, y1;
         hadamard_pair(arow[0], hmat, l, y0, y1);       // same wave wrote arow[0]: LDS operations of a wave stay in order
         uint16_t sc;
         const uint16_t q = quant_pair(y0, y1, sc);
-        const long long dst = p.k_cache_index[t];
         if (dst >= 0 && dst < p.cache_rows) {
             reinterpret_cast<uint16_t *>(p.k_cache + (size_t)dst * LIP_DIM)[l] = q;
             if (l == 0) p.k_cache_scale[dst] = sc;
@@ -416,13 +576,16 @@ hipError_t lip_launch(const LipParams &p, hipStream_t stream)
     const int steps = p.q_lora / LIP_KSPLIT / 32;
     const int tblocks = (p.T + 31) / 32;
     const int q_jobs = p.n_heads * LIP_KSPLIT * tblocks;
-    const int x_jobs = (p.h / LIP_XBLOCK) * ((p.T + 3) / 4);
-    const dim3 grid1((unsigned)(q_jobs + x_jobs)), block1(64);
-    const size_t lds = (size_t)steps * 32 * 128 + (size_t)steps * 1024;
+    const int x_jobs = 2 * (p.h / LIP_XBLOCK) * ((p.T + XTOK - 1) / XTOK);
+    // enough workgroups that each hidden-axis wave gets about one job, never fewer than the query jobs
+    int wgs = (x_jobs + LIN_XWAVES - 1) / LIN_XWAVES;
+    wgs = wgs > 4096 ? 4096 : wgs;
+    wgs = wgs > q_jobs ? wgs : q_jobs;
+    const dim3 grid1((unsigned)wgs), block1(128 + 64 * LIN_XWAVES);
     switch (steps) {
-    case 4: hipLaunchKernelGGL(lip_linear_kernel<4>, grid1, block1, lds, stream, p, q_jobs); break;
-    case 8: hipLaunchKernelGGL(lip_linear_kernel<8>, grid1, block1, lds, stream, p, q_jobs); break;
-    case 12: hipLaunchKernelGGL(lip_linear_kernel<12>, grid1, block1, lds, stream, p, q_jobs); break;
+    case 4: hipLaunchKernelGGL(lip_linear_kernel<2>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
+    case 8: hipLaunchKernelGGL(lip_linear_kernel<4>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
+    case 12: hipLaunchKernelGGL(lip_linear_kernel<6>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
     default: return hipErrorInvalidValue;
     }
     hipError_t e = hipGetLastError();
