@@ -80,3 +80,36 @@ def test_config4_prefill_4096_tokens(c_oracle):
     v = v.to(torch.bfloat16)
     assert torch.equal(out[0, 0].view(torch.int16), v.view(torch.int16).expand(128, 512)), "single-key row"
     check(out, golden(c_oracle, inp), "cfg4")
+
+
+def test_prolog_indexer_chain(c_oracle):
+    """Prolog -> indexer on the GPU against prolog oracle -> indexer oracle: the prolog's int8 query, fp16 scales
+    and weights and its freshly written key rows feed the indexer; the selected indices must be identical."""
+    from oracle import lip_oracle as lo
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs
+    K = 2048
+    act = [5000, 4097, 3000, 2049]
+    inp = gen_indexer_prolog_inputs(4, 2, act, seed=11)
+    inp.q_norm_scale *= 1e-3            # keeps fp16(q_scale * weight) of the indexer finite
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    t, n = 8, 64
+    dev = torch.device(DEV)
+    d = inp.to(dev)
+    q_int8 = torch.empty([t, n, 128], dtype=torch.int8, device=dev)
+    q_scale = torch.empty([t, n, 1], dtype=torch.float16, device=dev)
+    weights = torch.empty([t, n], dtype=torch.float16, device=dev)
+    pypto_amd.lightning_indexer_prolog_quant(*d.input_tensors(), q_int8, q_scale, d.k_cache, d.k_cache_scale, weights,
+                                             pypto_amd.IndexerPrologQuantAttr(), pypto_amd.IndexerPrologQuantConfigs())
+    act_t = torch.tensor(act, dtype=torch.int32)
+    res = torch.full([t, 1, K], -7, dtype=torch.int32, device=dev)
+    nb, bs = d.k_cache.shape[0], d.k_cache.shape[1]
+    pypto_amd.lightning_indexer_decode(q_int8, q_scale.reshape(t, n), d.k_cache, d.k_cache_scale.reshape(nb, bs, 1),
+                                       weights, act_t.to(dev), d.block_table, res, None, None, K)
+    torch.cuda.synchronize()
+    want = c_oracle.li_decode(torch.from_numpy(ref["q_int8"]), torch.from_numpy(ref["q_scale"]),
+                              torch.from_numpy(ref["k_cache"]), torch.from_numpy(ref["k_cache_scale"]).reshape(nb, bs, 1),
+                              torch.from_numpy(ref["weights"]), act_t, inp.block_table, K)
+    got = res.cpu()
+    assert torch.equal(got, want), f"{int((got != want).sum())} index mismatches"
+    # the last two positions of every sequence are the rows the prolog has just written: selectable
+    assert int((got >= 0).sum()) == sum(min(a - 1, K) + min(a, K) for a in act)
