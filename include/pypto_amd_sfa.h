@@ -35,6 +35,12 @@
  *       (examples/models/deepseek_v32_exp/lightning_indexer_prolog_quant_impl.py:507-562),
  *       same dispatch point: the projection stage that produces the indexer's
  *       int8 query, per-head weights and the new int8 key rows of the paged cache.
+ *   pto_mla_prolog_quant_launch
+ *       the device execution of mla_prolog_quant_d / _p
+ *       (examples/models/deepseek_v32_exp/mla_prolog_quant_impl.py:710-869), same
+ *       dispatch point: the projection stage that produces the attention's query
+ *       (absorbed nope part and rope part), the int8 query latent the indexer prolog
+ *       consumes, and the new rows of the latent / rope / scale caches.
  *   pto_*_workspace_bytes
  *       the workspace query the reference runtime performs before a launch
  *       (python/pypto/runtime.py:151-152, GetWorkSpaceSize).
@@ -274,6 +280,70 @@ typedef struct PtoLiPrologQuantArgs {
 
 int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *args, size_t *bytes);
 int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *args, void *hip_stream);
+
+/*
+ * MLA prolog, quantized (mla_prolog_quant_impl.py:502-707 in the reference example;
+ * torch golden deepseekv32_mla_prolog_quant.py:137-282), in the variant of the
+ * reference's enabled case: bf16 down-projections, int8 w_uq_qr with per-column
+ * scales, int8 latent cache with four fp32 scales per token, cache mode PA_BSND.
+ *
+ *   token_x        [t, h]                        bf16
+ *   w_dq           [h, q_lora_rank]              bf16   row-major
+ *   w_uq_qr        [q_lora_rank, n_heads*192]    int8   row-major; per head 128 nope + 64 rope columns
+ *   dequant_scale  [n_heads*192, 1]              fp32
+ *   w_uk           [n_heads, 128, 512]           bf16
+ *   w_dkv_kr       [h, 576]                      bf16   row-major; 512 latent + 64 rope columns
+ *   gamma_cq [q_lora_rank], gamma_ckv [512]      bf16
+ *   cos, sin       [t, 64]                       bf16
+ *   cache_index    [t]                           int64  physical cache row of each token
+ *   kv_cache       [block_num, block_size, 1, 512]  int8   rows cache_index[i] rewritten
+ *   kr_cache       [block_num, block_size, 1, 64]   bf16   same rows
+ *   k_scale_cache  [block_num, block_size, 1, 4]    fp32   same rows
+ *   q_norm_out         [t, q_lora_rank]          int8   written
+ *   q_norm_scale_out   [t, 1]                    fp32   written
+ *   query_nope_out     [t, n_heads, 512]         bf16   written
+ *   query_rope_out     [t, n_heads, 64]          bf16   written
+ *
+ * Every fp32 sum has a fixed order (hidden-axis sums as in the indexer prolog; RMS
+ * sums as a balanced tree over each slab of 128 channels, slabs ascending; the
+ * 128-term sums against w_uk ascending), so results are reproducible bit for bit.
+ * RMS norm: v / sqrt(mean(v^2) + epsilon) * gamma (epsilon 0 = the torch golden).
+ *
+ * Constraints: q_lora_rank in {512, 1024, 1536}, h a positive multiple of 64 up to
+ * 16384, n_heads even, t >= 1.
+ */
+typedef struct PtoMlaPrologQuantArgs {
+    const void *token_x;
+    const void *w_dq;
+    const int8_t *w_uq_qr;
+    const float *dequant_scale;
+    const void *w_uk;
+    const void *w_dkv_kr;
+    const void *gamma_cq;
+    const void *gamma_ckv;
+    const void *cos;
+    const void *sin;
+    const int64_t *cache_index;
+    int8_t *kv_cache;
+    void *kr_cache;
+    float *k_scale_cache;
+    int8_t *q_norm_out;
+    float *q_norm_scale_out;
+    void *query_nope_out;
+    void *query_rope_out;
+    void *workspace;
+    size_t workspace_bytes;
+    int64_t t;
+    int64_t h;
+    int64_t q_lora_rank;
+    int64_t n_heads;
+    int64_t cache_rows;   /* block_num * block_size */
+    float epsilon_cq;
+    float epsilon_ckv;
+} PtoMlaPrologQuantArgs;
+
+int pto_mla_prolog_quant_workspace_bytes(const PtoMlaPrologQuantArgs *args, size_t *bytes);
+int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *args, void *hip_stream);
 
 /* Thread-local description of the last error on this thread ("" if none). */
 const char *pto_last_error(void);

@@ -11,6 +11,7 @@
 
 #include "li_kernels.h"
 #include "lip_kernels.h"
+#include "mlap_kernels.h"
 #include "sfa_kernels.h"
 
 namespace {
@@ -220,6 +221,37 @@ size_t lip_ws_bytes(const PtoLiPrologQuantArgs *a)
     return lip_qpart_bytes(a) + (size_t)(a->h / pto::LIP_XBLOCK) * a->t * pto::LIP_XCOLS * sizeof(float);
 }
 
+int mlap_check(const PtoMlaPrologQuantArgs *a)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "mla_prolog: args is NULL");
+    if (a->t < 1 || a->t > (1ll << 20)) return fail(PTO_E_INVALID_ARG, "mla_prolog: t must be in [1, 2^20]");
+    if (a->n_heads < 2 || a->n_heads % 2 != 0 || a->n_heads > 1024)
+        return fail(PTO_E_INVALID_ARG, "mla_prolog: n_heads must be even, in [2, 1024] (got %lld)", (long long)a->n_heads);
+    if (a->q_lora_rank != 512 && a->q_lora_rank != 1024 && a->q_lora_rank != 1536)
+        return fail(PTO_E_INVALID_ARG, "mla_prolog: q_lora_rank must be 512, 1024 or 1536 (got %lld)", (long long)a->q_lora_rank);
+    const long long max_h = (long long)pto::MLAP_MAX_XGROUPS * pto::MLAP_XGROUP * pto::MLAP_XBLOCK;
+    if (a->h < pto::MLAP_XBLOCK || a->h % pto::MLAP_XBLOCK != 0 || a->h > max_h)
+        return fail(PTO_E_INVALID_ARG, "mla_prolog: h must be a positive multiple of %d, at most %lld (got %lld)", pto::MLAP_XBLOCK,
+                    max_h, (long long)a->h);
+    if (a->cache_rows < 1 || a->cache_rows > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "mla_prolog: cache_rows out of range");
+    if (!std::isfinite(a->epsilon_cq) || a->epsilon_cq < 0 || !std::isfinite(a->epsilon_ckv) || a->epsilon_ckv < 0)
+        return fail(PTO_E_INVALID_ARG, "mla_prolog: epsilons must be finite and >= 0");
+    return PTO_OK;
+}
+
+// [group sums over the hidden axis | 4 partial int32 projections]
+size_t mlap_xpart_bytes(const PtoMlaPrologQuantArgs *a)
+{
+    const size_t nblk = (size_t)a->h / pto::MLAP_XBLOCK;
+    const size_t ngroups = (nblk + pto::MLAP_XGROUP - 1) / pto::MLAP_XGROUP;
+    const size_t bytes = ngroups * a->t * (a->q_lora_rank + pto::MLAP_KV + pto::MLAP_ROPE) * sizeof(float);
+    return (bytes + 255) & ~(size_t)255;
+}
+size_t mlap_ws_bytes(const PtoMlaPrologQuantArgs *a)
+{
+    return mlap_xpart_bytes(a) + (size_t)pto::QPROJ_KSPLIT_HOST * a->t * a->n_heads * pto::MLAP_QHEAD * sizeof(int32_t);
+}
+
 }  // namespace
 
 extern "C" {
@@ -399,6 +431,67 @@ int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
     p.w_mul1 = (float)std::pow((double)pto::LIP_DIM, -0.5);
     hipError_t e = pto::lip_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li_prolog: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
+}
+
+int pto_mla_prolog_quant_workspace_bytes(const PtoMlaPrologQuantArgs *a, size_t *bytes)
+{
+    if (!bytes) return fail(PTO_E_INVALID_ARG, "mla_prolog: bytes is NULL");
+    int rc = mlap_check(a);
+    if (rc != PTO_OK) return rc;
+    *bytes = mlap_ws_bytes(a);
+    return PTO_OK;
+}
+
+int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream)
+{
+    int rc = mlap_check(a);
+    if (rc != PTO_OK) return rc;
+    const void *ptrs[] = {a->token_x, a->w_dq, a->w_uq_qr, a->dequant_scale, a->w_uk, a->w_dkv_kr, a->gamma_cq, a->gamma_ckv,
+                          a->cos, a->sin, a->cache_index, a->kv_cache, a->kr_cache, a->k_scale_cache, a->q_norm_out,
+                          a->q_norm_scale_out, a->query_nope_out, a->query_rope_out};
+    for (const void *ptr : ptrs)
+        if (!ptr) return fail(PTO_E_INVALID_ARG, "mla_prolog: a tensor pointer is NULL");
+    const size_t need = mlap_ws_bytes(a);
+    if (!a->workspace || a->workspace_bytes < need)
+        return fail(PTO_E_WORKSPACE, "mla_prolog: workspace of %zu bytes required, %zu given", need,
+                    a->workspace ? a->workspace_bytes : (size_t)0);
+    const void *aligned[] = {a->token_x, a->w_dq, a->w_uq_qr, a->dequant_scale, a->w_uk, a->w_dkv_kr, a->gamma_cq, a->gamma_ckv,
+                             a->kv_cache, a->k_scale_cache, a->q_norm_out, a->workspace};
+    for (const void *ptr : aligned)
+        if (reinterpret_cast<uintptr_t>(ptr) & 15)
+            return fail(PTO_E_INVALID_ARG, "mla_prolog: tensor and workspace pointers must be 16-byte aligned");
+
+    pto::MlapParams p;
+    p.x = static_cast<const uint16_t *>(a->token_x);
+    p.w_dq = static_cast<const uint16_t *>(a->w_dq);
+    p.w_uqqr = a->w_uq_qr;
+    p.w_qb_scale = a->dequant_scale;
+    p.w_uk = static_cast<const uint16_t *>(a->w_uk);
+    p.w_dkvkr = static_cast<const uint16_t *>(a->w_dkv_kr);
+    p.gamma_cq = static_cast<const uint16_t *>(a->gamma_cq);
+    p.gamma_ckv = static_cast<const uint16_t *>(a->gamma_ckv);
+    p.cos = static_cast<const uint16_t *>(a->cos);
+    p.sin = static_cast<const uint16_t *>(a->sin);
+    p.cache_index = reinterpret_cast<const long long *>(a->cache_index);
+    p.kv_cache = a->kv_cache;
+    p.kr_cache = static_cast<uint16_t *>(a->kr_cache);
+    p.k_scale_cache = a->k_scale_cache;
+    p.q_norm = a->q_norm_out;
+    p.q_norm_scale = a->q_norm_scale_out;
+    p.q_nope = static_cast<uint16_t *>(a->query_nope_out);
+    p.q_rope = static_cast<uint16_t *>(a->query_rope_out);
+    p.xpart = static_cast<float *>(a->workspace);
+    p.qpart = reinterpret_cast<int32_t *>(static_cast<char *>(a->workspace) + mlap_xpart_bytes(a));
+    p.cache_rows = a->cache_rows;
+    p.T = (int)a->t;
+    p.h = (int)a->h;
+    p.q_lora = (int)a->q_lora_rank;
+    p.n_heads = (int)a->n_heads;
+    p.eps_cq = a->epsilon_cq;
+    p.eps_ckv = a->epsilon_ckv;
+    hipError_t e = pto::mlap_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
 }
 

@@ -1,0 +1,47 @@
+// Launch parameters of the MLA prolog kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pto {
+
+constexpr int MLAP_NOPE = 128;       // query channels per head that meet w_uk
+constexpr int MLAP_ROPE = 64;        // rotated channels per head and of the key
+constexpr int MLAP_KV = 512;         // latent width
+constexpr int MLAP_QHEAD = MLAP_NOPE + MLAP_ROPE;
+constexpr int MLAP_XBLOCK = 64;      // block length of the fixed-order sums over the hidden axis
+constexpr int MLAP_XGROUP = 8;       // block sums per group (one workgroup of the first kernel)
+constexpr int MLAP_MAX_XGROUPS = 32; // h <= 32 * 8 * 64 = 16384
+constexpr int MLAP_MAX_QLORA = 1536;
+constexpr int QPROJ_KSPLIT_HOST = 4; // partial sums of the int8 projection (prolog_common.h: QPROJ_KSPLIT)
+constexpr int MLAP_XTOK = 8;         // tokens per job of the first and of the last kernel
+
+struct MlapParams {
+    const uint16_t *x;            // [T, h] bf16
+    const uint16_t *w_dq;         // [h, q_lora] bf16
+    const int8_t *w_uqqr;         // [q_lora, n_heads*192] int8
+    const float *w_qb_scale;      // [n_heads*192]
+    const uint16_t *w_uk;         // [n_heads, 128, 512] bf16
+    const uint16_t *w_dkvkr;      // [h, 576] bf16
+    const uint16_t *gamma_cq;     // [q_lora] bf16
+    const uint16_t *gamma_ckv;    // [512] bf16
+    const uint16_t *cos;          // [T, 64] bf16
+    const uint16_t *sin;          // [T, 64] bf16
+    const long long *cache_index; // [T]
+    int8_t *kv_cache;             // [cache_rows, 512]
+    uint16_t *kr_cache;           // [cache_rows, 64] bf16
+    float *k_scale_cache;         // [cache_rows, 4]
+    int8_t *q_norm;               // [T, q_lora]         written, then read by the projection
+    float *q_norm_scale;          // [T]
+    uint16_t *q_nope;             // [T, n_heads, 512] bf16
+    uint16_t *q_rope;             // [T, n_heads, 64] bf16
+    float *xpart;                 // workspace [ceil(h/512), T, q_lora + 576]
+    int32_t *qpart;               // workspace [4, T, n_heads*192]
+    long long cache_rows;
+    int T, h, q_lora, n_heads;
+    float eps_cq, eps_ckv;
+};
+
+hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
+
+}  // namespace pto

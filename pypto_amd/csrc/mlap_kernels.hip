@@ -1,0 +1,361 @@
+// MLA prolog for gfx950, the variant with bf16 down-projections, an int8 query up-projection and an
+// int8 latent cache with four fp32 scales per token: from a decode batch of hidden states it produces
+// the absorbed query (nope and rope parts), the int8 normalised query latent with its scale (input of
+// the indexer prolog), and writes the new latent / rope / scale rows of the paged caches.
+//
+// Arithmetic (reference golden: examples/models/deepseek_v32_exp/deepseekv32_mla_prolog_quant.py:137-282;
+// operator graph: examples/models/deepseek_v32_exp/mla_prolog_quant_impl.py:502-707).  Every fp32 sum
+// has a fixed order (all products are bf16 x bf16, exact in fp32): sums over the hidden axis in blocks of
+// 64 ascending, eight block sums ascending into a group sum, group sums ascending; the RMS sums as a
+// balanced tree over the 128 channels of a slab, slab sums ascending; the 128-term sums against w_uk
+// ascending.  Only the exact integer projection runs on the matrix cores.
+//
+// Four launches:
+//   mlap_xlinear_kernel  x . [w_dq | w_dkv_kr]: one workgroup of eight waves per (slab of 128 columns,
+//                        group of 512 hidden rows, 8 tokens); each wave takes a 64-row block (staged by
+//                        LDS-DMA, hidden states widened to fp32 in LDS), block sums meet in LDS and are
+//                        chained into the group sum.
+//   mlap_mid_kernel      per token: group sums chained, bf16, RMS norm (one wave per slab), per-token
+//                        int8 quantisation of the query latent; RMS norm and per-slab quantisation of
+//                        the key latent, rope of the key, scatter into the caches.
+//   qproj_kernel         int8 projection of the query latent (shared job code: LDS-DMA tile,
+//                        v_perm_b32 transposes, v_mfma_i32_32x32x32_i8), partial sums per quarter.
+//   mlap_finish_kernel   per (head, half of the 512 output columns, 8 tokens): partial sums added and
+//                        de-quantised, rope part rotated and stored, nope part times the head's w_uk
+//                        slice (staged in LDS by LDS-DMA), one output column per lane, 8 tokens at once.
+#include "mlap_kernels.h"
+#include "prolog_common.h"
+
+#pragma clang fp contract(off)
+
+namespace pto {
+namespace {
+
+static_assert(QPROJ_KSPLIT == QPROJ_KSPLIT_HOST, "workspace sizing and kernels disagree");
+
+constexpr int XL_WAVES = MLAP_XGROUP;                                  // one block per wave
+constexpr int XL_W_BYTES = MLAP_XBLOCK * 256;                          // a block of one slab: 64 rows x 256 bytes
+constexpr int XL_REGION = XL_W_BYTES + MLAP_XTOK * MLAP_XBLOCK * 4;    // + the hidden states as fp32
+
+// Column slabs: 0 .. q_lora/128 - 1 of w_dq, then four slabs of w_dkv_kr's latent part and one half slab
+// (64 columns) of its rope part.
+__global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapParams p, const int nslabs, const int ngroups)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XL_WAVES * XL_REGION];
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int slab = blockIdx.x % nslabs;
+    const int g = (blockIdx.x / nslabs) % ngroups;
+    const int t0 = (blockIdx.x / nslabs / ngroups) * MLAP_XTOK;
+    const int qslabs = p.q_lora / 128;
+    const int nblk = p.h / MLAP_XBLOCK;
+    const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
+    // the slab's matrix, row pitch and width in bytes
+    const bool isq = slab < qslabs;
+    const uint8_t *wbase = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256
+                               : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
+    const int pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
+    const int wbytes = (!isq && slab - qslabs == 4) ? 128 : 256;
+
+    uint8_t *region = smem + w * XL_REGION;
+    float *xs = reinterpret_cast<float *>(region + XL_W_BYTES);         // [8][64]
+    const int c = g * MLAP_XGROUP + w;                                    // this wave's block
+    const int nb = nblk - g * MLAP_XGROUP < MLAP_XGROUP ? nblk - g * MLAP_XGROUP : MLAP_XGROUP;
+    float a0[MLAP_XTOK], a1[MLAP_XTOK];
+#pragma unroll
+    for (int t = 0; t < MLAP_XTOK; ++t) a0[t] = a1[t] = 0.f;
+
+    if (w < nb) {
+        const int k0 = c * MLAP_XBLOCK;
+        const uint32_t wdst = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+        {   // rows of wbytes bytes: wbytes/16 lanes per row
+            const int lpr = wbytes >> 4;
+            const int rpi = 64 / lpr;                                     // rows per request
+            const uint8_t *src = wbase + (size_t)(k0 + l / lpr) * pitch + 16 * (l % lpr);
+#pragma unroll 1
+            for (int i = 0; i < MLAP_XBLOCK / rpi; ++i) dma16(src + (size_t)i * rpi * pitch, wdst + 1024 * i);
+        }
+#pragma unroll
+        for (int u = 0; u < MLAP_XTOK / 2; ++u) {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + 2u + l/32
+            const int t = t0 + 2 * u + (l >> 5);
+            const int tt = t < p.T ? t : p.T - 1;
+            const uint32_t xv = reinterpret_cast<const uint32_t *>(p.x + (size_t)tt * p.h + k0)[l & 31];
+            f32x2 v = {__uint_as_float(xv << 16), __uint_as_float(xv & 0xffff0000u)};
+            *reinterpret_cast<f32x2 *>(xs + (2 * u + (l >> 5)) * MLAP_XBLOCK + 2 * (l & 31)) = v;
+        }
+        VM_WAIT(0);
+        const uint32_t *wl = reinterpret_cast<const uint32_t *>(region) + (wbytes == 256 ? l : (l & 31));
+        const int rowdw = wbytes >> 2;
+#pragma unroll 1
+        for (int kk = 0; kk < MLAP_XBLOCK; kk += 4) {
+            f32x4 xv[MLAP_XTOK];
+#pragma unroll
+            for (int t = 0; t < MLAP_XTOK; ++t) xv[t] = *reinterpret_cast<const f32x4 *>(xs + t * MLAP_XBLOCK + kk);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t wv = wl[(kk + j) * rowdw];
+                const float w0 = __uint_as_float(wv << 16), w1 = __uint_as_float(wv & 0xffff0000u);
+#pragma unroll
+                for (int t = 0; t < MLAP_XTOK; ++t) {
+                    a0[t] = __builtin_fmaf(xv[t][j], w0, a0[t]);
+                    a1[t] = __builtin_fmaf(xv[t][j], w1, a1[t]);
+                }
+            }
+        }
+        // block sums into this wave's own (consumed) region: [8 tokens][128 columns]
+        float *bs = reinterpret_cast<float *>(region);
+#pragma unroll
+        for (int t = 0; t < MLAP_XTOK; ++t) {
+            f32x2 v = {a0[t], a1[t]};
+            *reinterpret_cast<f32x2 *>(bs + t * 128 + 2 * l) = v;
+        }
+    }
+    __syncthreads();
+    // group sum: thread (token = w, columns 2l, 2l+1) chains the block sums in ascending order
+    {
+        const int t = t0 + w;
+        const int width = wbytes >> 1;                                    // columns of the slab
+        if (t < p.T && 2 * l < width) {
+            float s0 = 0.f, s1 = 0.f;
+            for (int i = 0; i < nb; ++i) {
+                const f32x2 v = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(smem + i * XL_REGION) + w * 128 + 2 * l);
+                s0 = __fadd_rn(s0, v[0]);
+                s1 = __fadd_rn(s1, v[1]);
+            }
+            f32x2 v = {s0, s1};
+            *reinterpret_cast<f32x2 *>(p.xpart + ((size_t)g * p.T + t) * nc + slab * 128 + 2 * l) = v;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+constexpr int MID_WAVES = MLAP_MAX_QLORA / 128;   // 12
+
+// sum over the wave's 128 values of rn(rn(v*v) * coef) as a balanced tree over neighbours
+__device__ __forceinline__ float slab_square_sum(const float v0, const float v1, const float coef)
+{
+    return pair_tree_sum(__fmul_rn(__fmul_rn(v0, v0), coef), __fmul_rn(__fmul_rn(v1, v1), coef));
+}
+
+// Workgroup 2t: the query latent of token t (one wave per slab of 128 channels).  Workgroup 2t+1: its
+// key latent (waves 0..3) and key rope part (wave 4).
+__global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapParams p, const int ngroups)
+{
+    __shared__ float slabsum[MID_WAVES];
+    __shared__ float slabmax[MID_WAVES];
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t = blockIdx.x >> 1;
+    const bool kvtype = blockIdx.x & 1;
+    const int qslabs = p.q_lora / 128;
+    const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
+    const int nslab = kvtype ? 4 : qslabs;                               // slabs under the norm
+    const bool rope_wave = kvtype && w == 4;
+    const bool active = w < nslab || rope_wave;
+    const int col = (kvtype ? p.q_lora : 0) + w * 128 + 2 * (rope_wave ? (l & 31) : l);
+
+    float v0 = 0.f, v1 = 0.f;
+    if (active) {
+        const float *src = p.xpart + (size_t)t * nc + col;
+        for (int g = 0; g < ngroups; ++g) {
+            const f32x2 v = *reinterpret_cast<const f32x2 *>(src + (size_t)g * p.T * nc);
+            v0 = __fadd_rn(v0, v[0]);
+            v1 = __fadd_rn(v1, v[1]);
+        }
+        v0 = bf16_round_f32(v0);
+        v1 = bf16_round_f32(v1);
+    }
+    const long long dst = kvtype ? p.cache_index[t] : -1;
+    const bool dst_ok = dst >= 0 && dst < p.cache_rows;
+
+    if (rope_wave) {
+        // lane l < 32 holds channels 2l and 2l+1, which after the de-interleave are channels l and 32+l:
+        // the two partners of one rotation
+        if (l < 32) {
+            const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
+            const float s0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), s1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
+            const float r0 = __builtin_fmaf(v0, c0, (-v1) * s0);      // products exact: one rounding
+            const float r1 = __builtin_fmaf(v1, c1, v0 * s1);
+            if (dst_ok) {
+                p.kr_cache[(size_t)dst * MLAP_ROPE + l] = (uint16_t)(pack_bf16x2(r0, 0.f) & 0xffffu);
+                p.kr_cache[(size_t)dst * MLAP_ROPE + 32 + l] = (uint16_t)(pack_bf16x2(r1, 0.f) & 0xffffu);
+            }
+        }
+    }
+    const int n = kvtype ? MLAP_KV : p.q_lora;
+    if (w < nslab) {
+        const float ss = slab_square_sum(v0, v1, (float)(1.0 / (double)n));
+        if (l == 0) slabsum[w] = ss;
+    }
+    __syncthreads();
+    float y0 = 0.f, y1 = 0.f;
+    if (w < nslab) {
+        float s = 0.f;
+        for (int j = 0; j < nslab; ++j) s = __fadd_rn(s, slabsum[j]);
+        const float d = __fsqrt_rn(__fadd_rn(s, kvtype ? p.eps_ckv : p.eps_cq));
+        const uint32_t gm = reinterpret_cast<const uint32_t *>(kvtype ? p.gamma_ckv : p.gamma_cq)[w * 64 + l];
+        y0 = bf16_round_f32(__fmul_rn(__fdiv_rn(v0, d), __uint_as_float(gm << 16)));
+        y1 = bf16_round_f32(__fmul_rn(__fdiv_rn(v1, d), __uint_as_float(gm & 0xffff0000u)));
+        const float m = wave_max_f32(fmaxf(fabsf(y0), fabsf(y1)));
+        if (l == 0) slabmax[w] = m;
+    }
+    __syncthreads();
+    if (w < nslab) {
+        float amax = slabmax[w];
+        if (!kvtype)
+            for (int j = 0; j < nslab; ++j) amax = fmaxf(amax, slabmax[j]);
+        float deq;
+        const uint16_t q = quant_pair_amax(y0, y1, amax, deq);
+        if (!kvtype) {
+            reinterpret_cast<uint16_t *>(p.q_norm + (size_t)t * p.q_lora)[w * 64 + l] = q;
+            if (w == 0 && l == 0) p.q_norm_scale[t] = deq;
+        } else if (dst_ok) {
+            reinterpret_cast<uint16_t *>(p.kv_cache + (size_t)dst * MLAP_KV)[w * 64 + l] = q;
+            if (l == 0) p.k_scale_cache[(size_t)dst * 4 + w] = deq;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int HS>
+__global__ __launch_bounds__(128) void qproj_kernel(const QProj p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * lin_region_bytes<HS>()];
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l = threadIdx.x & 63;
+    const int job = blockIdx.x;
+    uint8_t *region = smem + w * lin_region_bytes<HS>();
+    i32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+    q_half_job<HS>(p, region, job, w, acc);
+    if (w == 1) q_pair_park(region, l, acc);
+    __syncthreads();
+    if (w == 0) q_pair_store<HS>(p, smem, job, l, acc);
+}
+
+// ---------------------------------------------------------------------------------------------
+constexpr int FIN_W_BYTES = MLAP_NOPE * 64 * 2;    // a wave's slice of w_uk[head]: 128 rows x 64 columns bf16
+
+// Workgroup (head, half of the 512 output columns, block of 8 tokens); wave w owns output columns
+// colbase + 64w + l.
+__global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t wsl[4 * FIN_W_BYTES];
+    __shared__ __attribute__((aligned(16))) float arow[MLAP_XTOK][MLAP_NOPE];
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int head = blockIdx.x % p.n_heads;
+    const int half = (blockIdx.x / p.n_heads) & 1;
+    const int t0 = (blockIdx.x / p.n_heads / 2) * MLAP_XTOK;
+    const int ncols = p.n_heads * MLAP_QHEAD;
+    const int colbase = half * 256 + 64 * w;
+
+    {   // this wave's slice: rows of 128 bytes, pitch 1024 bytes: 8 lanes per row, 8 rows per request
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(p.w_uk) + ((size_t)head * MLAP_NOPE + (l >> 3)) * (MLAP_KV * 2) +
+                             colbase * 2 + 16 * (l & 7);
+        const uint32_t dst = (uint32_t)(uintptr_t)(lds_byte_t *)(wsl + w * FIN_W_BYTES);
+#pragma unroll 1
+        for (int i = 0; i < MLAP_NOPE / 8; ++i) dma16(src + (size_t)i * 8 * MLAP_KV * 2, dst + 1024 * i);
+    }
+    // the head's query channels of tokens t0 + w and t0 + 4 + w: partial sums added, de-quantised, bf16
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int tl = 4 * u + w;
+        const int t = t0 + tl;
+        const int tt = t < p.T ? t : p.T - 1;
+        const float ts = p.q_norm_scale[tt];
+        // nope part: lane l -> channels 2l, 2l+1
+        {
+            const int col = head * MLAP_QHEAD + 2 * l;
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
+                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + tt) * ncols + col);
+                s0 += v.x;
+                s1 += v.y;
+            }
+            const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
+            f32x2 av = {bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0])),
+                        bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]))};
+            *reinterpret_cast<f32x2 *>(&arow[tl][2 * l]) = av;
+        }
+        // rope part (first half-workgroup only): lane l < 32 -> channels 2l, 2l+1 = rotation partners l, 32+l
+        if (half == 0 && l < 32 && t < p.T) {
+            const int col = head * MLAP_QHEAD + MLAP_NOPE + 2 * l;
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
+                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + t) * ncols + col);
+                s0 += v.x;
+                s1 += v.y;
+            }
+            const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
+            const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
+            const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
+            const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
+            const float sn0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), sn1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
+            const float r0 = __builtin_fmaf(v0, c0, (-v1) * sn0);
+            const float r1 = __builtin_fmaf(v1, c1, v0 * sn1);
+            uint16_t *out = p.q_rope + ((size_t)t * p.n_heads + head) * MLAP_ROPE;
+            out[l] = (uint16_t)(pack_bf16x2(r0, 0.f) & 0xffffu);
+            out[32 + l] = (uint16_t)(pack_bf16x2(r1, 0.f) & 0xffffu);
+        }
+    }
+    VM_WAIT(0);
+    __syncthreads();
+
+    // out[t][colbase + 64w + l] = sum_i a[t][i] * w_uk[head][i][col], i ascending; 8 tokens at once
+    const uint16_t *wl = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) + l;
+    float acc[MLAP_XTOK];
+#pragma unroll
+    for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = 0.f;
+#pragma unroll 2
+    for (int i = 0; i < MLAP_NOPE; i += 4) {
+        f32x4 av[MLAP_XTOK];
+#pragma unroll
+        for (int t = 0; t < MLAP_XTOK; ++t) av[t] = *reinterpret_cast<const f32x4 *>(&arow[t][i]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float wv = bf16_bits_to_f32(wl[(i + j) * 64]);
+#pragma unroll
+            for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = __builtin_fmaf(av[t][j], wv, acc[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < MLAP_XTOK; ++t)
+        if (t0 + t < p.T)
+            p.q_nope[((size_t)(t0 + t) * p.n_heads + head) * MLAP_KV + colbase + l] = (uint16_t)(pack_bf16x2(acc[t], 0.f) & 0xffffu);
+}
+
+}  // namespace
+
+hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
+{
+    const int nblk = p.h / MLAP_XBLOCK;
+    const int ngroups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
+    const int nslabs = p.q_lora / 128 + 5;
+    const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
+    hipLaunchKernelGGL(mlap_xlinear_kernel, dim3((unsigned)(nslabs * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, nslabs, ngroups);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(mlap_mid_kernel, dim3((unsigned)(2 * p.T)), dim3(64 * MID_WAVES), 0, stream, p, ngroups);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128};
+    const dim3 qgrid((unsigned)(qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32)));
+    switch (p.q_lora / QPROJ_KSPLIT / 32) {
+    case 4: hipLaunchKernelGGL(qproj_kernel<2>, qgrid, dim3(128), 0, stream, qp); break;
+    case 8: hipLaunchKernelGGL(qproj_kernel<4>, qgrid, dim3(128), 0, stream, qp); break;
+    case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp); break;
+    default: return hipErrorInvalidValue;
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)(p.n_heads * 2 * tgroups)), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace pto

@@ -1,0 +1,231 @@
+// Device helpers shared by the two prolog kernels files (lightning-indexer prolog, MLA prolog):
+// explicit vector-memory waits, the int8 projection job (row-major int8 weight tile -> LDS by LDS-DMA
+// -> v_mfma_i32_32x32x32_i8), fp32 wave reductions in a fixed order without LDS traffic.
+#pragma once
+#include "common.h"
+
+namespace pto {
+namespace {
+
+constexpr int QPROJ_KSPLIT = 4;     // jobs that share the reduction axis of the int8 projection
+
+struct QProj {
+    const int8_t *q_norm;   // [T, q_lora]
+    const int8_t *w;        // [q_lora, 128 * nslabs], row-major
+    int32_t *part;          // [QPROJ_KSPLIT, T, 128 * nslabs]
+    int T, q_lora, nslabs;
+};
+
+#define VM_WAIT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | (((n) >> 4) << 14) | 0x0F70))
+
+// at most n (a multiple of 4, <= 60) vector-memory requests of this wave still outstanding
+__device__ __forceinline__ void wait_vm_le(const int n)
+{
+    switch (n) {
+    case 4: VM_WAIT(4); break;
+    case 8: VM_WAIT(8); break;
+    case 12: VM_WAIT(12); break;
+    case 16: VM_WAIT(16); break;
+    case 20: VM_WAIT(20); break;
+    case 24: VM_WAIT(24); break;
+    case 28: VM_WAIT(28); break;
+    case 32: VM_WAIT(32); break;
+    case 36: VM_WAIT(36); break;
+    case 40: VM_WAIT(40); break;
+    case 44: VM_WAIT(44); break;
+    default: VM_WAIT(0); break;
+    }
+}
+
+// rows d0..d3 of four bytes each -> columns o0..o3 (o_i = byte i of d0, d1, d2, d3)
+__device__ __forceinline__ void transpose4x4(const uint32_t d0, const uint32_t d1, const uint32_t d2, const uint32_t d3,
+                                             uint32_t &o0, uint32_t &o1, uint32_t &o2, uint32_t &o3)
+{
+    const uint32_t t0 = __builtin_amdgcn_perm(d1, d0, 0x05010400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);
+    const uint32_t u0 = __builtin_amdgcn_perm(d3, d2, 0x05010400u);
+    const uint32_t u1 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
+    o0 = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
+    o1 = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
+    o2 = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
+    o3 = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
+}
+
+__device__ __forceinline__ float bf16_round_f32(const float v)
+{
+    return __uint_as_float(pack_bf16x2(v, 0.0f) << 16);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Int8 projection [T, q_lora] x [q_lora, 128*nslabs] -> partial int32 sums: one job per (slab of 128 columns, quarter of the reduction axis, block of 32 tokens); its
+// waves 0 and 1 take one half of the quarter each (HS steps of 32 rows).
+// LDS region of a wave: [tile: 32*HS rows x 128 bytes][token operands: HS x 1024 bytes].
+// Matrix product per step: A = 32 output columns x 32 rows of the tile (lane (j, g) holds rows
+// 16g..16g+15 of column 4j+i for product i), B = 32 tokens x the same 32 rows of q_norm, so that
+// accumulator register r of lane l holds column 4*(8*(r/4) + 4*(l/32) + r%4) + i, token l%32.
+template <int HS>
+__device__ __forceinline__ void q_half_job(const QProj &p, uint8_t *region, const int job, const int half, i32x16 (&acc)[4])
+{
+    const int l = threadIdx.x & 63;
+    const int ncols = p.nslabs * 128;
+    const int kq = job & (QPROJ_KSPLIT - 1);
+    const int head = (job >> 2) % p.nslabs;
+    const int tb = (job >> 2) / p.nslabs;
+    constexpr int KH = HS * 32;                        // rows of this wave
+    constexpr int NW = KH / 8;                         // tile requests of 8 rows each
+    const int k0 = (kq * 2 + half) * KH;
+    const uint32_t tile = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+    const uint32_t tok = tile + KH * 128;
+
+    // token operands and the tile: every request is issued before the first wait.  The loops stay
+    // rolled: straight-line code that runs once is bound by instruction fetch.
+    {
+        int t = tb * 32 + (l & 31);
+        t = t < p.T ? t : p.T - 1;
+        const int8_t *src = p.q_norm + (size_t)t * p.q_lora + k0 + 16 * (l >> 5);
+#pragma unroll 1
+        for (int s = 0; s < HS; ++s) dma16(src + 32 * s, tok + 1024 * s);
+    }
+    {
+        const int8_t *src = p.w + ((size_t)k0 + (l >> 3)) * ncols + head * 128 + 16 * (l & 7);
+#pragma unroll 2
+        for (int i = 0; i < NW; ++i) dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
+    }
+    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(region);
+    const int rd = (16 * (l >> 5)) * 32 + (l & 31);     // dword index of this lane's first row of a step
+    // The tile arrives at the pace of the memory system; each step starts as soon as its four
+    // requests have landed (requests complete in order), so only the last step trails the arrival.
+#pragma unroll
+    for (int s = 0; s < HS; ++s) {
+        wait_vm_le(NW - 4 * (s + 1));
+        uint32_t d[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
+        const i32x4 b = *reinterpret_cast<const i32x4 *>(region + KH * 128 + 1024 * s + 16 * l);
+        i32x4 a[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            uint32_t o0, o1, o2, o3;
+            transpose4x4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3], o0, o1, o2, o3);
+            a[0][q] = (int)o0;
+            a[1][q] = (int)o1;
+            a[2][q] = (int)o2;
+            a[3][q] = (int)o3;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+    }
+}
+
+constexpr int LIN_RED_BYTES = 16 * 64 * 16;           // one wave's accumulators, 16 bytes per (register, lane)
+
+template <int HS>
+constexpr int lin_region_bytes()
+{
+    return HS * (32 * 128 + 1024) > LIN_RED_BYTES ? HS * (32 * 128 + 1024) : LIN_RED_BYTES;
+}
+
+// Both halves done (the caller has passed a workgroup barrier since wave 1 wrote its accumulators to
+// its region): wave 0 adds them to its own and stores the partial sums of its 32 tokens x 128 columns.
+template <int HS>
+__device__ __forceinline__ void q_pair_store(const QProj &p, const uint8_t *smem, const int job, const int l, const i32x16 (&acc)[4])
+{
+    const i32x4 *red = reinterpret_cast<const i32x4 *>(smem + lin_region_bytes<HS>());
+    const int ncols = p.nslabs * 128;
+    const int kq = job & (QPROJ_KSPLIT - 1);
+    const int head = (job >> 2) % p.nslabs;
+    const int t = ((job >> 2) / p.nslabs) * 32 + (l & 31);
+    if (t < p.T) {
+        int32_t *dst = p.part + ((size_t)kq * p.T + t) * ncols + head * 128;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
+            const i32x4 o = red[r * 64 + l];
+            i32x4 v = {acc[0][r] + o[0], acc[1][r] + o[1], acc[2][r] + o[2], acc[3][r] + o[3]};
+            *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
+        }
+    }
+}
+// wave 1 parks its accumulators in its own (consumed) tile region
+__device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const i32x16 (&acc)[4])
+{
+    i32x4 *red = reinterpret_cast<i32x4 *>(region);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        red[r * 64 + l] = v;
+    }
+}
+
+// Cross-lane exchanges without LDS traffic.  dpp_f32 reads another lane of the same row of 16;
+// row_swap16 / half_swap32 return {own-side, other-side} copies across rows of 16 / halves of 32
+// (v_permlane16_swap, v_permlane32_swap with both operands equal).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(const float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+constexpr int DPP_XOR1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int DPP_XOR2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141;  // lane i of a group of 8 reads lane 7-i
+constexpr int DPP_MIRROR = 0x140;     // lane i of a row of 16 reads lane 15-i
+
+// value held by lane l ^ 16
+__device__ __forceinline__ float xor16_f32(const float v, const int l)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    // r[0]: rows 0,0,2,2 of v;  r[1]: rows 1,1,3,3
+    return __uint_as_float((l & 16) ? r[0] : r[1]);
+}
+
+// combine(own, partner) over the whole wave where combine is commutative and every step leaves all
+// lanes of the finished group with the same bits: xor 1, xor 2, then mirrors within 8 and 16 lanes
+// (the mirrored lane lies in the other half, which is uniform), then the row and half swaps.
+#define WAVE_BUTTERFLY(v, OP)                                                                              \
+    do {                                                                                                   \
+        v = OP(v, dpp_f32<DPP_XOR1>(v));                                                                   \
+        v = OP(v, dpp_f32<DPP_XOR2>(v));                                                                   \
+        v = OP(v, dpp_f32<DPP_HALF_MIRROR>(v));                                                            \
+        v = OP(v, dpp_f32<DPP_MIRROR>(v));                                                                 \
+        {                                                                                                  \
+            const auto r_ = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false); \
+            v = OP(__uint_as_float(r_[0]), __uint_as_float(r_[1]));                                        \
+        }                                                                                                  \
+        {                                                                                                  \
+            const auto r_ = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false); \
+            v = OP(__uint_as_float(r_[0]), __uint_as_float(r_[1]));                                        \
+        }                                                                                                  \
+    } while (0)
+
+__device__ __forceinline__ float wave_max_f32(float v)
+{
+    WAVE_BUTTERFLY(v, fmaxf);
+    return v;
+}
+
+// sum of the wave's 128 values (two per lane, neighbours) as a balanced tree over neighbours
+__device__ __forceinline__ float pair_tree_sum(const float v0, const float v1)
+{
+    float s = __fadd_rn(v0, v1);
+    WAVE_BUTTERFLY(s, __fadd_rn);
+    return s;
+}
+
+
+// symmetric int8 quantisation of two values per lane against a given maximum of magnitudes; returns
+// the packed byte pair and the de-quantisation scale (both 0 when the maximum is 0)
+__device__ __forceinline__ uint16_t quant_pair_amax(const float y0, const float y1, const float amax, float &deq)
+{
+    if (amax > 0.f) {
+        const float s = __fdiv_rn(127.0f, amax);
+        const int q0 = (int)rintf(__fmul_rn(y0, s));
+        const int q1 = (int)rintf(__fmul_rn(y1, s));
+        deq = __fdiv_rn(1.0f, s);
+        return (uint16_t)((q0 & 0xff) | ((q1 & 0xff) << 8));
+    }
+    deq = 0.f;
+    return 0;
+}
+
+}  // namespace
+}  // namespace pto

@@ -229,4 +229,54 @@ PYBIND11_MODULE(_C, m)
               a.eps = static_cast<float>(eps);
               check(pto_li_prolog_quant_launch(&a, ptr<void>(stream)));
           });
+
+    m.def("mla_prolog_quant_workspace_bytes", [](int64_t t, int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows) {
+        PtoMlaPrologQuantArgs a{};
+        a.t = t;
+        a.h = h;
+        a.q_lora_rank = q_lora_rank;
+        a.n_heads = n_heads;
+        a.cache_rows = cache_rows;
+        size_t bytes = 0;
+        check(pto_mla_prolog_quant_workspace_bytes(&a, &bytes));
+        return bytes;
+    });
+    m.def("mla_prolog_quant_launch",
+          [](std::uintptr_t token_x, std::uintptr_t w_dq, std::uintptr_t w_uq_qr, std::uintptr_t dequant_scale, std::uintptr_t w_uk,
+             std::uintptr_t w_dkv_kr, std::uintptr_t gamma_cq, std::uintptr_t gamma_ckv, std::uintptr_t cos, std::uintptr_t sin,
+             std::uintptr_t cache_index, std::uintptr_t kv_cache, std::uintptr_t kr_cache, std::uintptr_t k_scale_cache,
+             std::uintptr_t q_norm_out, std::uintptr_t q_norm_scale_out, std::uintptr_t query_nope_out,
+             std::uintptr_t query_rope_out, std::uintptr_t workspace, size_t workspace_bytes, int64_t t, int64_t h,
+             int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows, double epsilon_cq, double epsilon_ckv,
+             std::uintptr_t stream) {
+              PtoMlaPrologQuantArgs a{};
+              a.token_x = ptr<const void>(token_x);
+              a.w_dq = ptr<const void>(w_dq);
+              a.w_uq_qr = ptr<const int8_t>(w_uq_qr);
+              a.dequant_scale = ptr<const float>(dequant_scale);
+              a.w_uk = ptr<const void>(w_uk);
+              a.w_dkv_kr = ptr<const void>(w_dkv_kr);
+              a.gamma_cq = ptr<const void>(gamma_cq);
+              a.gamma_ckv = ptr<const void>(gamma_ckv);
+              a.cos = ptr<const void>(cos);
+              a.sin = ptr<const void>(sin);
+              a.cache_index = ptr<const int64_t>(cache_index);
+              a.kv_cache = ptr<int8_t>(kv_cache);
+              a.kr_cache = ptr<void>(kr_cache);
+              a.k_scale_cache = ptr<float>(k_scale_cache);
+              a.q_norm_out = ptr<int8_t>(q_norm_out);
+              a.q_norm_scale_out = ptr<float>(q_norm_scale_out);
+              a.query_nope_out = ptr<void>(query_nope_out);
+              a.query_rope_out = ptr<void>(query_rope_out);
+              a.workspace = ptr<void>(workspace);
+              a.workspace_bytes = workspace_bytes;
+              a.t = t;
+              a.h = h;
+              a.q_lora_rank = q_lora_rank;
+              a.n_heads = n_heads;
+              a.cache_rows = cache_rows;
+              a.epsilon_cq = static_cast<float>(epsilon_cq);
+              a.epsilon_ckv = static_cast<float>(epsilon_ckv);
+              check(pto_mla_prolog_quant_launch(&a, ptr<void>(stream)));
+          });
 }

@@ -14,6 +14,8 @@ the reference tree):
 * ``gen_indexer_prolog_inputs`` ...deepseekv32_lightning_indexer_prolog_quant.py:100-153
   (value ranges, tensor names and shapes; ``cache_index`` names the last ``s1``
   positions of every sequence, :76-84)
+* ``gen_mla_prolog_inputs`` ...deepseekv32_mla_prolog_quant.py:329-453 for ``is_quant = (False, True)``
+  (bf16 down-projections, per-channel int8 ``w_uqqr`` with its fp32 scales, value ranges)
 
 Unlike the reference (global ``torch.manual_seed`` plus an unseeded
 ``np.random.permutation``) every generator here draws from an explicit
@@ -290,6 +292,80 @@ def gen_indexer_prolog_inputs(b: int, s1: int, act_seq: Sequence[int], seed: int
                                wk=wk, w_proj=w_proj, ln_gamma_k=gamma, ln_beta_k=beta, cos_idx_rope=cos,
                                sin_idx_rope=sin, hadamard_q=hq, hadamard_k=hk, k_cache=k_cache,
                                k_cache_scale=k_cache_scale, k_cache_index=idx.reshape(t), block_table=table)
+
+
+@dataclass
+class MlaPrologInputs:
+    b: int
+    s1: int
+    block_size: int
+    block_num: int
+    act_seq: List[int]
+    token_x: torch.Tensor        # [T, h]                       bf16
+    w_dq: torch.Tensor           # [h, q_lora_rank]             bf16
+    w_uq_qr: torch.Tensor        # [q_lora_rank, N*192]         int8
+    dequant_scale: torch.Tensor  # [N*192, 1]                   fp32
+    w_uk: torch.Tensor           # [N, 128, 512]                bf16
+    w_dkv_kr: torch.Tensor       # [h, 576]                     bf16
+    gamma_cq: torch.Tensor       # [q_lora_rank]                bf16
+    gamma_ckv: torch.Tensor      # [512]                        bf16
+    cos: torch.Tensor            # [T, 64]                      bf16
+    sin: torch.Tensor            # [T, 64]                      bf16
+    cache_index: torch.Tensor    # [T]                          int64
+    kv_cache: torch.Tensor       # [NB, bs, 1, 512]             int8   (updated in place)
+    kr_cache: torch.Tensor       # [NB, bs, 1, 64]              bf16   (updated in place)
+    k_scale_cache: torch.Tensor  # [NB, bs, 1, 4]               fp32   (updated in place)
+    block_table: torch.Tensor    # [B, MB]                      int32
+
+    def input_tensors(self):
+        return (self.token_x, self.w_dq, self.w_uq_qr, self.dequant_scale, self.w_uk, self.w_dkv_kr, self.gamma_cq,
+                self.gamma_ckv, self.cos, self.sin, self.cache_index, self.kv_cache, self.kr_cache, self.k_scale_cache)
+
+    def to(self, device) -> "MlaPrologInputs":
+        kw = dict(self.__dict__)
+        for k, v in kw.items():
+            if isinstance(v, torch.Tensor):
+                kw[k] = v.to(device)
+        return MlaPrologInputs(**kw)
+
+
+def gen_mla_prolog_inputs(b: int, s1: int, act_seq: Sequence[int], seed: int = 0, h: int = 7168,
+                          q_lora_rank: int = 1536, n_heads: int = 128, block_size: int = BLOCK_SIZE) -> MlaPrologInputs:
+    """Value ranges of the reference generator: x, gammas uniform in (-1, 1), weights in (-0.1, 0.1) (w_uqqr
+    quantised per output channel to int8), cos/sin in (-0.1, 0.1); caches filled with random rows."""
+    g = torch.Generator().manual_seed(seed)
+    act = [int(a) for a in act_seq]
+    t = b * s1
+    bf = torch.bfloat16
+    d_nope, d_rope, kv_rank = 128, ROPE_DIM, KV_LORA_RANK
+
+    def uni(shape, lim, dtype):
+        return ((torch.rand(shape, generator=g, dtype=torch.float32) * 2 - 1) * lim).to(dtype)
+
+    x = uni([t, h], 1.0, bf)
+    w_dq = uni([h, q_lora_rank], 0.1, bf)
+    wq = uni([q_lora_rank, n_heads * (d_nope + d_rope)], 0.1, torch.float32)
+    amax = wq.abs().amax(dim=0, keepdim=True)
+    sq = 127.0 / amax
+    w_uq_qr = torch.round(wq * sq).to(torch.int8)
+    dequant_scale = (1.0 / sq).reshape(-1, 1).contiguous()
+    w_uk = uni([n_heads, d_nope, kv_rank], 0.1, bf)
+    w_dkv_kr = uni([h, kv_rank + d_rope], 0.1, bf)
+    gamma_cq, gamma_ckv = uni([q_lora_rank], 1.0, bf), uni([kv_rank], 1.0, bf)
+    cos, sin = uni([t, d_rope], 0.1, bf), uni([t, d_rope], 0.1, bf)
+    block_num, table = gen_block_table(act, block_size, g, shuffle=True)
+    kv_cache = torch.randint(-127, 128, [block_num, block_size, 1, kv_rank], generator=g, dtype=torch.int8)
+    kr_cache = uni([block_num, block_size, 1, d_rope], 1.0, bf)
+    k_scale_cache = 0.005 + 0.015 * torch.rand([block_num, block_size, 1, 4], generator=g, dtype=torch.float32)
+    idx = torch.empty([b, s1], dtype=torch.int64)
+    for i in range(b):
+        for j in range(s1):
+            pos = act[i] - s1 + j
+            idx[i, j] = int(table[i, pos // block_size]) * block_size + pos % block_size
+    return MlaPrologInputs(b=b, s1=s1, block_size=block_size, block_num=block_num, act_seq=act, token_x=x, w_dq=w_dq,
+                           w_uq_qr=w_uq_qr, dequant_scale=dequant_scale, w_uk=w_uk, w_dkv_kr=w_dkv_kr,
+                           gamma_cq=gamma_cq, gamma_ckv=gamma_ckv, cos=cos, sin=sin, cache_index=idx.reshape(t),
+                           kv_cache=kv_cache, kr_cache=kr_cache, k_scale_cache=k_scale_cache, block_table=table)
 
 
 def config_lengths(cfg: int, seed: int = 0) -> List[int]:

@@ -30,6 +30,7 @@ def test_header_symbols_are_exported(lib):
     names = _declared()
     assert {"pto_sfa_quant_launch", "pto_sfa_quant_workspace_bytes", "pto_li_decode_launch",
             "pto_li_decode_workspace_bytes", "pto_li_prolog_quant_launch", "pto_li_prolog_quant_workspace_bytes",
+            "pto_mla_prolog_quant_launch", "pto_mla_prolog_quant_workspace_bytes",
             "pto_last_error", "pto_version"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
@@ -59,6 +60,12 @@ def test_pybind_workspace_and_argument_errors():
         C.li_prolog_quant_workspace_bytes(8, 7100, 1536, 64, 1 << 20)                # h not a multiple of 64
     with pytest.raises(ValueError):
         C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 65, 1 << 20)                # more than 64 heads
+    # MLA prolog: 14 group sums [t, 1536 + 576] fp32 + 4 int32 partial projections [t, 128 * 192]
+    assert C.mla_prolog_quant_workspace_bytes(8, 7168, 1536, 128, 1 << 16) == 14 * 8 * 2112 * 4 + 4 * 8 * 24576 * 4
+    with pytest.raises(ValueError):
+        C.mla_prolog_quant_workspace_bytes(8, 7168, 1536, 127, 1 << 16)              # odd head count
+    with pytest.raises(ValueError):
+        C.mla_prolog_quant_workspace_bytes(8, 32768, 1536, 128, 1 << 16)             # hidden size beyond the limit
     with pytest.raises(ValueError):
         C.sfa_quant_workspace_bytes(1, 1, 128, 2, 2048, 128, 32, 4096, 0.04, 0)      # n_kv != 1
     with pytest.raises(ValueError):

@@ -1,0 +1,103 @@
+"""Parity of the HIP MLA prolog (through the operator, pybind11 and the C ABI) against the CPU oracle.  The
+oracle fixes the order of every fp32 sum, so the bar is bit-exact for every output: int8 query latent and
+its fp32 scale, bf16 absorbed query (nope and rope parts), and every byte of the three caches."""
+import numpy as np
+import pytest
+import torch
+
+import pypto_amd
+from oracle import mlap_oracle as mo
+from pypto_amd.synthetic import gen_mla_prolog_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def run_op(inp, eps=(0.0, 0.0), separate_cache_out=False, prefill=False):
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    t, n, ql = d.token_x.shape[0], d.w_uk.shape[0], d.w_dq.shape[1]
+    q_norm = torch.full([t, ql], -7, dtype=torch.int8, device=dev)
+    q_norm_scale = torch.full([t, 1], -7.0, dtype=torch.float32, device=dev)
+    q_nope = torch.full([t, n, 512], -7.0, dtype=torch.bfloat16, device=dev)
+    q_rope = torch.full([t, n, 64], -7.0, dtype=torch.bfloat16, device=dev)
+    if separate_cache_out:
+        kv, kr, ks = torch.zeros_like(d.kv_cache), torch.zeros_like(d.kr_cache), torch.zeros_like(d.k_scale_cache)
+    else:
+        kv, kr, ks = d.kv_cache, d.kr_cache, d.k_scale_cache
+    ins = [pypto_amd.from_torch(v) for v in d.input_tensors()]
+    outs = [pypto_amd.from_torch(v) for v in (q_norm, q_norm_scale, q_nope, q_rope, kv, kr, ks)]
+    fn = pypto_amd.mla_prolog_quant_p if prefill else pypto_amd.mla_prolog_quant_d
+    ret = fn(*ins, *outs, eps[0], eps[1], "PA_BSND", pypto_amd.MlaTileConfig(), pypto_amd.RopeTileShapeConfig())
+    assert ret is None
+    torch.cuda.synchronize()
+    return {"q_norm": q_norm.cpu().numpy(), "q_norm_scale": q_norm_scale.cpu().numpy()[:, 0],
+            "query_nope": q_nope.float().cpu().numpy(), "query_rope": q_rope.float().cpu().numpy(),
+            "kv_cache": kv.cpu().numpy(), "kr_cache": kr.float().cpu().numpy(), "k_scale_cache": ks.cpu().numpy()}
+
+
+def assert_exact(got, ref, what):
+    for name in ("q_norm", "q_norm_scale", "query_nope", "query_rope", "kv_cache", "kr_cache", "k_scale_cache"):
+        g, r = got[name], ref[name]
+        assert g.shape == r.shape, (what, name, g.shape, r.shape)
+        gi = g.view(np.uint8) if g.dtype == np.int8 else g.view(np.uint32)
+        ri = r.view(np.uint8) if r.dtype == np.int8 else r.view(np.uint32)
+        if not np.array_equal(gi, ri):
+            bad = np.argwhere(gi != ri)
+            first = tuple(bad[0])
+            raise AssertionError(f"{what}: {name}: {len(bad)} of {g.size} differ; first at {first}: got {g[first]} want {r[first]}")
+
+
+@pytest.mark.parametrize("b,s1,act,kw,eps", [
+    (2, 2, [300, 129], dict(h=256, q_lora_rank=512, n_heads=4), (0.0, 0.0)),        # small everything, golden's norm
+    (1, 1, [77], dict(h=1152, q_lora_rank=1024, n_heads=2), (1e-5, 1e-5)),          # one token, ragged last group (18 blocks)
+    (3, 1, [5, 128, 129], dict(h=512, q_lora_rank=1536, n_heads=8), (1e-5, 1e-6)),
+    (5, 7, [900] * 5, dict(h=192, q_lora_rank=512, n_heads=2), (1e-5, 1e-5)),       # 35 tokens: ragged groups of 8, two token blocks
+])
+def test_mla_prolog_small_shapes_bit_exact(b, s1, act, kw, eps):
+    inp = gen_mla_prolog_inputs(b, s1, act, seed=3 * b + s1, **kw)
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=eps[0], epsilon_ckv=eps[1])
+    assert_exact(run_op(inp, eps), ref, f"b={b} s1={s1} {kw}")
+
+
+def test_mla_prolog_reference_case_b4_s2():
+    """Shapes of the reference's enabled test (deepseekv32_mla_prolog_quant.py:790-834): b=4, s=2, 128 heads,
+    h=7168, q_lora_rank=1536, epsilons 1e-5 as its driver passes them."""
+    inp = gen_mla_prolog_inputs(4, 2, [4096] * 4, seed=0)
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    got = run_op(inp, (1e-5, 1e-5))
+    assert_exact(got, ref, "b4_s2")
+    # and the reference's own acceptance rule against the library-order evaluation of its golden
+    qn, qs, qnope, qrope, ki, kr, ks = mo.mla_prolog_library_order(*inp.input_tensors()[:10])
+    rows = inp.cache_index.numpy()
+    assert np.abs(got["q_norm"].astype(np.int32) - qn.numpy().astype(np.int32)).max() <= 1
+    assert np.abs(got["q_norm_scale"] - qs.numpy()).max() <= 2.5e-5 + 0.005 * np.abs(qs.numpy()).max()
+    for g, r in ((got["query_nope"], qnope.float().numpy()), (got["query_rope"], qrope.float().numpy())):
+        assert (np.abs(g - r) > 0.005 + 0.0078125 * np.abs(r)).mean() <= 0.005
+    assert np.abs(got["kv_cache"].reshape(-1, 512)[rows].astype(np.int32) - ki.numpy().astype(np.int32)).max() <= 1
+    assert np.abs(got["kr_cache"].reshape(-1, 64)[rows] - kr.float().numpy()).max() <= 1e-4 + 0.0078125 * np.abs(kr.float().numpy()).max()
+    assert np.abs(got["k_scale_cache"].reshape(-1, 4)[rows] - ks.numpy()).max() <= 2.5e-5 + 0.005 * np.abs(ks.numpy()).max()
+
+
+def test_mla_prolog_separate_cache_output_skipped_indices_and_repeatability():
+    inp = gen_mla_prolog_inputs(2, 2, [300, 129], seed=5, h=256, q_lora_rank=512, n_heads=4)
+    inp.cache_index[1] = -1
+    inp.cache_index[2] = inp.kv_cache.shape[0] * inp.kv_cache.shape[1]
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    a = run_op(inp, (1e-5, 1e-5), separate_cache_out=True, prefill=True)
+    assert_exact(a, ref, "separate outputs, two skipped indices")
+    assert_exact(run_op(inp, (1e-5, 1e-5), separate_cache_out=True), a, "second run")
+
+
+def test_mla_prolog_feeds_the_attention_cache_layout():
+    """The rows the prolog writes are the rows the attention reads: int8 latent, four fp32 scales, bf16 rope,
+    at the page-table position of the newest tokens.  De-quantising them reproduces the normalised latent."""
+    inp = gen_mla_prolog_inputs(2, 1, [200, 131], seed=8, h=256, q_lora_rank=512, n_heads=2)
+    got = run_op(inp, (1e-5, 1e-5))
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    table = inp.block_table.numpy()
+    for bi, a in enumerate(inp.act_seq):
+        row = table[bi, (a - 1) // 128] * 128 + (a - 1) % 128
+        assert row == int(inp.cache_index[bi])
+        deq = got["kv_cache"].reshape(-1, 512)[row].astype(np.float32).reshape(4, 128) * got["k_scale_cache"].reshape(-1, 4)[row][:, None]
+        np.testing.assert_array_equal(got["kv_cache"].reshape(-1, 512)[row], ref["k_int8"][bi])
+        assert np.abs(deq.reshape(512)).max() > 0
