@@ -17,6 +17,7 @@ timed region.  Prints ONE JSON line:
   indexer_prolog time of one lightning-indexer prolog pass (projection stage) on the reference's enabled
                  case b=4, s1=2 (8 tokens, h=7168, q_lora_rank=1536), launches replayed from a HIP graph so
                  that host time between launches is not counted, with its HBM fraction
+  mla_prolog     the same for the MLA prolog (b=4, s=2, 128 heads; 85 MB of weights per pass, ten sets)
   cpu_baseline   the scalar C statement of the golden, all host threads, on a bounded sample of the
                  same batch
 
@@ -139,6 +140,53 @@ def prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=20, replays=10):
             "bytes": byt, "hbm_frac": byt / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
 
 
+def mla_prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=10, replays=10):
+    """One MLA prolog pass = the four launches of mla_prolog_quant_d; timed like prolog_leg (HIP graph of `calls`
+    passes, each with its own copy of the four weight tensors: 10 x 85 MB exceeds the memory-side cache)."""
+    from pypto_amd.synthetic import gen_mla_prolog_inputs
+    d = gen_mla_prolog_inputs(b, s1, [4096] * b, seed=0).to(dev)
+    t, n, ql, h = b * s1, d.w_uk.shape[0], d.w_dq.shape[1], d.token_x.shape[1]
+    outs = (torch.empty([t, ql], dtype=torch.int8, device=dev), torch.empty([t, 1], dtype=torch.float32, device=dev),
+            torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev), torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev),
+            d.kv_cache, d.kr_cache, d.k_scale_cache)
+    ins = list(d.input_tensors())
+    sets = [(ins[1].clone(), ins[2].clone(), ins[4].clone(), ins[5].clone()) for _ in range(calls)]
+
+    def one(i=0):
+        a = list(ins)
+        a[1], a[2], a[4], a[5] = sets[i]
+        pypto_amd.mla_prolog_quant_d(*a, *outs, 1e-5, 1e-5, "PA_BSND", None, None)
+    for _ in range(3):
+        one()
+    torch.cuda.synchronize()
+    mode = "hip graph replay"
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(calls):
+                one(i)
+        run = g.replay
+    except Exception:                      # noqa: BLE001 -- capture support varies; eager timing still valid
+        mode = "eager calls (host time included)"
+
+        def run():
+            for i in range(calls):
+                one(i)
+    run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (calls * replays)
+    byt = h * ql * 2 + ql * n * 192 + n * 128 * 512 * 2 + h * 576 * 2 + t * (h * 2 + ql + n * 576 * 2 + 656)
+    return {"workload": f"b={b} s={s1} (t={t}) h={h} q_lora_rank={ql} {n} heads", "us_per_pass": us,
+            "timing": mode + f", {calls} weight sets in rotation", "bytes": byt,
+            "hbm_frac": byt / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -259,6 +307,7 @@ def main():
 
     # ------------------------------------------------------------------ indexer prolog (projection stage)
     prolog = prolog_leg(torch, dev, pypto_amd)
+    mla_prolog = mla_prolog_leg(torch, dev, pypto_amd)
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
@@ -309,6 +358,7 @@ def main():
                     "configs[1]_us_per_step": li1_avg_ms * 1e3, "configs[1]_hbm_frac": li1_bytes / (li1_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes, "scale_dtype": "fp32", "weight_dtype": "bf16"},
         "indexer_prolog": prolog,
+        "mla_prolog": mla_prolog,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))

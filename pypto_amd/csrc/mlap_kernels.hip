@@ -86,7 +86,7 @@ __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapP
         VM_WAIT(0);
         const uint32_t *wl = reinterpret_cast<const uint32_t *>(region) + (wbytes == 256 ? l : (l & 31));
         const int rowdw = wbytes >> 2;
-#pragma unroll 1
+#pragma unroll 2
         for (int kk = 0; kk < MLAP_XBLOCK; kk += 4) {
             f32x4 xv[MLAP_XTOK];
 #pragma unroll
@@ -217,23 +217,49 @@ __global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapPara
 }
 
 // ---------------------------------------------------------------------------------------------
+// One workgroup (two waves, one half of a quarter tile each) walks the jobs blockIdx.x, + gridDim.x, ...:
+// the tile of the next job is requested into the other buffer before the current one is consumed, so the
+// weights stream without a gap between jobs.  The wave pair adds its accumulators through one of two
+// parking areas, alternating, with one barrier per job.
 template <int HS>
-__global__ __launch_bounds__(128) void qproj_kernel(const QProj p)
+constexpr int qproj_lds_bytes()
 {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * lin_region_bytes<HS>()];
+    return 4 * HS * (32 * 128 + 1024) + 2 * LIN_RED_BYTES;
+}
+
+template <int HS>
+__global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njobs)
+{
+    constexpr int BUF = HS * (32 * 128 + 1024);
+    constexpr int NREQ = HS * 5;                       // requests of one job per wave
+    __shared__ __attribute__((aligned(16))) uint8_t smem[qproj_lds_bytes<HS>()];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = threadIdx.x & 63;
-    const int job = blockIdx.x;
-    uint8_t *region = smem + w * lin_region_bytes<HS>();
-    i32x16 acc[4];
+    uint8_t *bufs = smem + w * 2 * BUF;
+    uint8_t *park = smem + 4 * BUF;
+    int job = blockIdx.x;
+    if (job < njobs) q_issue<HS>(p, bufs, job, w);
+    for (int k = 0; job < njobs; job += gridDim.x, ++k) {
+        const int next = job + gridDim.x;
+        if (next < njobs) {
+            q_issue<HS>(p, bufs + ((k + 1) & 1) * BUF, next, w);
+            VM_WAIT(NREQ);
+        } else {
+            VM_WAIT(0);
+        }
+        i32x16 acc[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
-    q_half_job<HS>(p, region, job, w, acc);
-    if (w == 1) q_pair_park(region, l, acc);
-    __syncthreads();
-    if (w == 0) q_pair_store<HS>(p, smem, job, l, acc);
+            for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+        const uint8_t *region = bufs + (k & 1) * BUF;
+#pragma unroll 1
+        for (int s = 0; s < HS; ++s) q_step<HS>(region, s, l, acc);
+        uint8_t *pk = park + (k & 1) * LIN_RED_BYTES;
+        if (w == 1) q_pair_park(pk, l, acc);
+        __syncthreads();
+        if (w == 0) q_pair_store_from(p, pk, job, l, acc);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -307,27 +333,56 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
     VM_WAIT(0);
     __syncthreads();
 
-    // out[t][colbase + 64w + l] = sum_i a[t][i] * w_uk[head][i][col], i ascending; 8 tokens at once
+    // out[t][colbase + 64w + l] = sum_i a[t][i] * w_uk[head][i][col], i ascending; 8 tokens at once.
+    // Chunks of four rows are read one chunk ahead of the multiply-adds that consume them.
     const uint16_t *wl = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) + l;
     float acc[MLAP_XTOK];
 #pragma unroll
     for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = 0.f;
-#pragma unroll 2
-    for (int i = 0; i < MLAP_NOPE; i += 4) {
-        f32x4 av[MLAP_XTOK];
+    struct Chunk {
+        f32x4 a[MLAP_XTOK];
+        uint16_t w[4];
+    };
+    auto load = [&](Chunk &c, const int i) {
 #pragma unroll
-        for (int t = 0; t < MLAP_XTOK; ++t) av[t] = *reinterpret_cast<const f32x4 *>(&arow[t][i]);
+        for (int t = 0; t < MLAP_XTOK; ++t) c.a[t] = *reinterpret_cast<const f32x4 *>(&arow[t][i]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c.w[j] = wl[(i + j) * 64];
+    };
+    auto fma = [&](const Chunk &c) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float wv = bf16_bits_to_f32(wl[(i + j) * 64]);
+            const float wv = bf16_bits_to_f32(c.w[j]);
 #pragma unroll
-            for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = __builtin_fmaf(av[t][j], wv, acc[t]);
+            for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = __builtin_fmaf(c.a[t][j], wv, acc[t]);
         }
+    };
+    Chunk c0, c1;
+    load(c0, 0);
+#pragma unroll 1
+    for (int i = 0; i < MLAP_NOPE; i += 8) {
+        load(c1, i + 4);
+        fma(c0);
+        load(c0, i + 8 < MLAP_NOPE ? i + 8 : 0);
+        fma(c1);
     }
 #pragma unroll
     for (int t = 0; t < MLAP_XTOK; ++t)
         if (t0 + t < p.T)
             p.q_nope[((size_t)(t0 + t) * p.n_heads + head) * MLAP_KV + colbase + l] = (uint16_t)(pack_bf16x2(acc[t], 0.f) & 0xffffu);
+}
+
+int cu_count()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cached = n;
+        else
+            cached = 256;
+    }
+    return cached;
 }
 
 }  // namespace
@@ -345,11 +400,17 @@ hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128};
-    const dim3 qgrid((unsigned)(qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32)));
-    switch (p.q_lora / QPROJ_KSPLIT / 32) {
-    case 4: hipLaunchKernelGGL(qproj_kernel<2>, qgrid, dim3(128), 0, stream, qp); break;
-    case 8: hipLaunchKernelGGL(qproj_kernel<4>, qgrid, dim3(128), 0, stream, qp); break;
-    case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp); break;
+    const int qjobs = qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);
+    // as many workgroups as fit at once (by their LDS), every one with the same number of jobs where possible
+    const int steps = p.q_lora / QPROJ_KSPLIT / 32;
+    const int lds = steps == 12 ? qproj_lds_bytes<6>() : (steps == 8 ? qproj_lds_bytes<4>() : qproj_lds_bytes<2>());
+    const int slots = cu_count() * (160 * 1024 / lds);
+    const int rounds = (qjobs + slots - 1) / slots;
+    const dim3 qgrid((unsigned)((qjobs + rounds - 1) / rounds));
+    switch (steps) {
+    case 4: hipLaunchKernelGGL(qproj_kernel<2>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
+    case 8: hipLaunchKernelGGL(qproj_kernel<4>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
+    case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
     default: return hipErrorInvalidValue;
     }
     e = hipGetLastError();

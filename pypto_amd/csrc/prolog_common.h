@@ -64,7 +64,7 @@ __device__ __forceinline__ float bf16_round_f32(const float v)
 // 16g..16g+15 of column 4j+i for product i), B = 32 tokens x the same 32 rows of q_norm, so that
 // accumulator register r of lane l holds column 4*(8*(r/4) + 4*(l/32) + r%4) + i, token l%32.
 template <int HS>
-__device__ __forceinline__ void q_half_job(const QProj &p, uint8_t *region, const int job, const int half, i32x16 (&acc)[4])
+__device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const int job, const int half)
 {
     const int l = threadIdx.x & 63;
     const int ncols = p.nslabs * 128;
@@ -91,29 +91,45 @@ __device__ __forceinline__ void q_half_job(const QProj &p, uint8_t *region, cons
 #pragma unroll 2
         for (int i = 0; i < NW; ++i) dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
     }
+}
+
+// one 32-row step of the product from the wave's region
+template <int HS>
+__device__ __forceinline__ void q_step(const uint8_t *region, const int s, const int l, i32x16 (&acc)[4])
+{
+    constexpr int KH = HS * 32;
     const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(region);
     const int rd = (16 * (l >> 5)) * 32 + (l & 31);     // dword index of this lane's first row of a step
-    // The tile arrives at the pace of the memory system; each step starts as soon as its four
-    // requests have landed (requests complete in order), so only the last step trails the arrival.
+    uint32_t d[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
+    const i32x4 b = *reinterpret_cast<const i32x4 *>(region + KH * 128 + 1024 * s + 16 * l);
+    i32x4 a[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t o0, o1, o2, o3;
+        transpose4x4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3], o0, o1, o2, o3);
+        a[0][q] = (int)o0;
+        a[1][q] = (int)o1;
+        a[2][q] = (int)o2;
+        a[3][q] = (int)o3;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+}
+
+// A single job: issue, then every step as soon as its four requests have landed (requests complete
+// in order), so only the last step trails the arrival of the tile.
+template <int HS>
+__device__ __forceinline__ void q_half_job(const QProj &p, uint8_t *region, const int job, const int half, i32x16 (&acc)[4])
+{
+    constexpr int NW = HS * 4;
+    q_issue<HS>(p, region, job, half);
+    const int l = threadIdx.x & 63;
 #pragma unroll
     for (int s = 0; s < HS; ++s) {
         wait_vm_le(NW - 4 * (s + 1));
-        uint32_t d[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
-        const i32x4 b = *reinterpret_cast<const i32x4 *>(region + KH * 128 + 1024 * s + 16 * l);
-        i32x4 a[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            uint32_t o0, o1, o2, o3;
-            transpose4x4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3], o0, o1, o2, o3);
-            a[0][q] = (int)o0;
-            a[1][q] = (int)o1;
-            a[2][q] = (int)o2;
-            a[3][q] = (int)o3;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+        q_step<HS>(region, s, l, acc);
     }
 }
 
@@ -125,12 +141,11 @@ constexpr int lin_region_bytes()
     return HS * (32 * 128 + 1024) > LIN_RED_BYTES ? HS * (32 * 128 + 1024) : LIN_RED_BYTES;
 }
 
-// Both halves done (the caller has passed a workgroup barrier since wave 1 wrote its accumulators to
-// its region): wave 0 adds them to its own and stores the partial sums of its 32 tokens x 128 columns.
-template <int HS>
-__device__ __forceinline__ void q_pair_store(const QProj &p, const uint8_t *smem, const int job, const int l, const i32x16 (&acc)[4])
+// Both halves done (the caller has passed a workgroup barrier since wave 1 parked its accumulators at
+// `parked`): wave 0 adds them to its own and stores the partial sums of its 32 tokens x 128 columns.
+__device__ __forceinline__ void q_pair_store_from(const QProj &p, const uint8_t *parked, const int job, const int l, const i32x16 (&acc)[4])
 {
-    const i32x4 *red = reinterpret_cast<const i32x4 *>(smem + lin_region_bytes<HS>());
+    const i32x4 *red = reinterpret_cast<const i32x4 *>(parked);
     const int ncols = p.nslabs * 128;
     const int kq = job & (QPROJ_KSPLIT - 1);
     const int head = (job >> 2) % p.nslabs;
@@ -145,6 +160,12 @@ __device__ __forceinline__ void q_pair_store(const QProj &p, const uint8_t *smem
             *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
         }
     }
+}
+// the same with wave 1's accumulators parked in its own (consumed) tile region, the second of two
+template <int HS>
+__device__ __forceinline__ void q_pair_store(const QProj &p, const uint8_t *smem, const int job, const int l, const i32x16 (&acc)[4])
+{
+    q_pair_store_from(p, smem + lin_region_bytes<HS>(), job, l, acc);
 }
 // wave 1 parks its accumulators in its own (consumed) tile region
 __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const i32x16 (&acc)[4])

@@ -113,3 +113,71 @@ def test_prolog_indexer_chain(c_oracle):
     assert torch.equal(got, want), f"{int((got != want).sum())} index mismatches"
     # the last two positions of every sequence are the rows the prolog has just written: selectable
     assert int((got >= 0).sum()) == sum(min(a - 1, K) + min(a, K) for a in act)
+
+
+def test_whole_decode_front_mla_prolog_indexer_prolog_indexer_attention(c_oracle):
+    """One decode step of the whole path on the GPU: MLA prolog -> indexer prolog (fed with the MLA prolog's int8
+    query latent) -> indexer (over the key rows just written) -> sparse attention (over the latent rows just
+    written, with the absorbed query), against the same chain of CPU oracles.  Every intermediate is bit-exact;
+    the attention output meets the attention tolerance."""
+    from oracle import lip_oracle as lo
+    from oracle import mlap_oracle as mo
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
+    B, S1, K, N = 4, 1, 2048, 128
+    act = [5000, 4097, 3000, 2049]
+    T = B * S1
+    mla = gen_mla_prolog_inputs(B, S1, act, seed=21)
+    lip = gen_indexer_prolog_inputs(B, S1, act, seed=22)
+    lip.x = mla.token_x                                   # one hidden state feeds both prologs
+    # one page table for all caches
+    lip.block_table, lip.k_cache_index = mla.block_table, mla.cache_index
+    nb, bs = mla.kv_cache.shape[0], mla.kv_cache.shape[1]
+    assert lip.k_cache.shape[0] == nb
+
+    # ---- CPU chain
+    r_mla = mo.mla_prolog_ref(*mla.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    lip_args = list(lip.input_tensors())
+    lip_args[1] = torch.from_numpy(r_mla["q_norm"])
+    lip_args[2] = torch.from_numpy(r_mla["q_norm_scale"]).reshape(T, 1) * 1e-3      # keeps the indexer's fp16 products finite
+    r_lip = lo.indexer_prolog_ref(*lip_args)
+    act_t = torch.tensor(act, dtype=torch.int32)
+    want_idx = c_oracle.li_decode(torch.from_numpy(r_lip["q_int8"]), torch.from_numpy(r_lip["q_scale"]),
+                                  torch.from_numpy(r_lip["k_cache"]), torch.from_numpy(r_lip["k_cache_scale"]).reshape(nb, bs, 1),
+                                  torch.from_numpy(r_lip["weights"]), act_t, mla.block_table, K)
+    qn = torch.from_numpy(r_mla["query_nope"]).to(torch.bfloat16).reshape(T * N, 512)
+    qr = torch.from_numpy(r_mla["query_rope"]).to(torch.bfloat16).reshape(T * N, 64)
+    kn = torch.from_numpy(r_mla["kv_cache"]).reshape(nb * bs, 512)
+    kr = torch.from_numpy(r_mla["kr_cache"]).to(torch.bfloat16).reshape(nb * bs, 64)
+    ks = torch.from_numpy(r_mla["k_scale_cache"]).reshape(nb * bs, 4)
+    scale = 576 ** -0.5
+    want_out = c_oracle.sfa_quant(qn, qr, kn, kr, ks, want_idx.reshape(T, K), mla.block_table, act_t, B, S1, N, K, bs,
+                                  scale, s2_tile=0)
+
+    # ---- GPU chain
+    dev = torch.device(DEV)
+    dm, dl = mla.to(dev), lip.to(dev)
+    q_norm = torch.empty([T, 1536], dtype=torch.int8, device=dev)
+    q_norm_scale = torch.empty([T, 1], dtype=torch.float32, device=dev)
+    q_nope = torch.empty([T, N, 512], dtype=torch.bfloat16, device=dev)
+    q_rope = torch.empty([T, N, 64], dtype=torch.bfloat16, device=dev)
+    pypto_amd.mla_prolog_quant_d(*dm.input_tensors(), q_norm, q_norm_scale, q_nope, q_rope, dm.kv_cache, dm.kr_cache,
+                                 dm.k_scale_cache, 1e-5, 1e-5, "PA_BSND", None, None)
+    q_int8 = torch.empty([T, 64, 128], dtype=torch.int8, device=dev)
+    q_scale = torch.empty([T, 64, 1], dtype=torch.float16, device=dev)
+    weights = torch.empty([T, 64], dtype=torch.float16, device=dev)
+    gl = list(dl.input_tensors())
+    gl[1], gl[2] = q_norm, q_norm_scale * 1e-3
+    pypto_amd.lightning_indexer_prolog_quant(*gl, q_int8, q_scale, dl.k_cache, dl.k_cache_scale, weights)
+    res = torch.empty([T, 1, K], dtype=torch.int32, device=dev)
+    pypto_amd.lightning_indexer_decode(q_int8, q_scale.reshape(T, 64), dl.k_cache, dl.k_cache_scale.reshape(nb, bs, 1),
+                                       weights, act_t.to(dev), dm.block_table, res, None, None, K)
+    out = torch.full([B, S1, N, 512], float("nan"), dtype=torch.bfloat16, device=dev)
+    pypto_amd.sparse_flash_attention_quant_d(q_nope.reshape(T * N, 512), q_rope.reshape(T * N, 64),
+                                             dm.kv_cache.reshape(nb * bs, 512), dm.kr_cache.reshape(nb * bs, 64),
+                                             dm.k_scale_cache.reshape(nb * bs, 4), res.reshape(T, K), dm.block_table,
+                                             act_t.to(dev), out, N, 1, scale, K, bs, dm.block_table.shape[1], None)
+    torch.cuda.synchronize()
+    assert torch.equal(q_norm.cpu(), torch.from_numpy(r_mla["q_norm"]))
+    assert torch.equal(q_int8.cpu(), torch.from_numpy(r_lip["q_int8"]))
+    assert torch.equal(res.cpu(), want_idx), f"{int((res.cpu() != want_idx).sum())} index mismatches"
+    check(out.cpu(), want_out, "whole decode front")
