@@ -101,3 +101,45 @@ def test_mla_prolog_feeds_the_attention_cache_layout():
         deq = got["kv_cache"].reshape(-1, 512)[row].astype(np.float32).reshape(4, 128) * got["k_scale_cache"].reshape(-1, 4)[row][:, None]
         np.testing.assert_array_equal(got["kv_cache"].reshape(-1, 512)[row], ref["k_int8"][bi])
         assert np.abs(deq.reshape(512)).max() > 0
+
+
+def test_fused_mla_indexer_prolog_matches_the_oracle_chain():
+    """mla_indexer_prolog_quant_d: the indexer prolog consumes the MLA prolog's hidden q_norm / q_norm_scale; the
+    ten outputs equal the two oracles chained (cos/sin of the MLA generator's range feed both stages)."""
+    from oracle import lip_oracle as lo
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs
+    kw = dict(h=256, q_lora_rank=512)
+    mla = gen_mla_prolog_inputs(2, 2, [300, 129], seed=14, n_heads=4, **kw)
+    lip = gen_indexer_prolog_inputs(2, 2, [300, 129], seed=15, n_heads=4, **kw)
+    assert lip.k_cache.shape[0] == mla.kv_cache.shape[0]
+    r_mla = mo.mla_prolog_ref(*mla.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    la = list(lip.input_tensors())
+    la[0], la[1], la[2] = mla.token_x, torch.from_numpy(r_mla["q_norm"]), torch.from_numpy(r_mla["q_norm_scale"]).reshape(-1, 1)
+    la[9], la[10], la[15] = mla.cos, mla.sin, mla.cache_index
+    r_lip = lo.indexer_prolog_ref(*la)
+
+    dev = torch.device("cuda:0")
+    dm, dl = mla.to(dev), lip.to(dev)
+    t, n = 4, 4
+    q_nope = torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev)
+    q_rope = torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev)
+    q_int8 = torch.empty([t, n, 128], dtype=torch.int8, device=dev)
+    q_scale = torch.empty([t, n, 1], dtype=torch.float16, device=dev)
+    weights = torch.empty([t, n], dtype=torch.float16, device=dev)
+    ret = pypto_amd.mla_indexer_prolog_quant_d(
+        dm.token_x, dm.w_dq, dm.w_uq_qr, dm.dequant_scale, dm.w_uk, dm.w_dkv_kr, dm.gamma_cq, dm.gamma_ckv, dm.cos, dm.sin,
+        dm.cache_index, dm.kv_cache, dm.kr_cache, dm.k_scale_cache, dl.w_qb, dl.w_qb_scale, dl.wk, dl.w_proj, dl.ln_gamma_k,
+        dl.ln_beta_k, dl.hadamard_q, dl.hadamard_k, dl.k_cache, dl.k_cache_scale, q_nope, q_rope, dm.kv_cache, dm.kr_cache,
+        dm.k_scale_cache, q_int8, q_scale, dl.k_cache, dl.k_cache_scale, weights, 1e-5, 1e-5, "PA_BSND",
+        pypto_amd.MlaTileConfig(), pypto_amd.IndexerPrologQuantAttr(), pypto_amd.IndexerPrologQuantConfigs(),
+        pypto_amd.RopeTileShapeConfig())
+    assert ret is None
+    torch.cuda.synchronize()
+    assert np.array_equal(q_nope.float().cpu().numpy(), r_mla["query_nope"])
+    assert np.array_equal(q_rope.float().cpu().numpy(), r_mla["query_rope"])
+    assert np.array_equal(dm.kv_cache.cpu().numpy(), r_mla["kv_cache"])
+    assert np.array_equal(q_int8.cpu().numpy(), r_lip["q_int8"])
+    assert np.array_equal(q_scale.cpu().numpy()[..., 0].view(np.uint16), r_lip["q_scale"].view(np.uint16))
+    assert np.array_equal(weights.cpu().numpy().view(np.uint16), r_lip["weights"].view(np.uint16))
+    assert np.array_equal(dl.k_cache.cpu().numpy(), r_lip["k_cache"])
+    assert np.array_equal(dl.k_cache_scale.cpu().numpy().view(np.uint16), r_lip["k_cache_scale"].view(np.uint16))
