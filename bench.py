@@ -200,7 +200,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
-              "(sharding over GPUs is described in DESIGN.md, not implemented)", file=sys.stderr)
+              "(query rows shard over GPUs without any exchange; that is not implemented here)", file=sys.stderr)
         sys.exit(2)
 
     import torch
