@@ -208,7 +208,11 @@ typedef struct PtoLiDecodeArgs {
     int32_t q_scale_dtype;
     int32_t k_scale_dtype;
     int32_t weight_dtype;
-    int32_t reserved;
+    int32_t arith_variant;   /* 0: the arithmetic above.  1: that of the reference's chained C++ operator
+                                (framework/src/operator/models/deepseek_v3.2_exp/lightning_indexer.cpp:149-197):
+                                v = fp16(q.k / 2048); v = fp16(fp16(v * q_scale) * k_scale); v = max(v, 0);
+                                v = fp16(v * weight); score = fp32 sum over heads, h ascending.  All three
+                                dtype codes must be PTO_DT_FP16. */
 } PtoLiDecodeArgs;
 
 int pto_li_decode_workspace_bytes(const PtoLiDecodeArgs *args, size_t *bytes);

@@ -56,6 +56,8 @@ __all__ = [
     "qk_relu_fp16",
     "head_sum",
     "li_scores",
+    "li_scores_fp16_dequant",
+    "lightning_indexer_fp16_dequant_ref",
     "canonical_topk",
     "lightning_indexer_ref",
 ]
@@ -122,6 +124,69 @@ def li_scores(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weig
             wq = head_sum(w_scale[t], x)
             rows.append((wq * ks_sel).astype(np.float32))
     return rows
+
+
+def li_scores_fp16_dequant(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight,
+                           act_seq_key: Sequence[int], block_table, s1: int | None = None) -> list[np.ndarray]:
+    """Score rows in the arithmetic of the reference's chained C++ operator (golden:
+    framework/tests/st/operator/src/test_deepseek_v3.2_exp/gen_lightning_indexer.py:243-257; graph:
+    framework/src/operator/models/deepseek_v3.2_exp/lightning_indexer.cpp:183-191), all scales and weights fp16:
+
+        v = fp16(float32(dot) * 2**-11)        signed
+        v = fp16(fp16(v * q_scale[h]) * k_scale[j])
+        v = max(v, 0);  v = fp16(v * weight[h])
+        score[j] = sum_h float32(v)            fp32, h ascending (the golden's torch.sum leaves the order open)
+
+    A product of two fp16 values is exact in fp32, so numpy's float16 multiply (computed in fp32, rounded once) is
+    the correctly rounded fp16 product."""
+    q = _np(idx_query)
+    t_tot, nh, d = q.shape
+    bt = _np(block_table)
+    b = len(act_seq_key)
+    if s1 is None:
+        s1 = t_tot // b
+    key = _np(idx_key_cache).reshape(-1, d)
+    bs = idx_key_cache.shape[1]
+    assert idx_query_scale.dtype == idx_key_scale.dtype == idx_weight.dtype == torch.float16
+    ks = idx_key_scale.reshape(-1).numpy()
+    qs = idx_query_scale.reshape(t_tot, nh).numpy()
+    wt = idx_weight.reshape(t_tot, nh).numpy()
+    rows = []
+    for b_idx in range(b):
+        cur = int(act_seq_key[b_idx])
+        pos = np.arange(cur, dtype=np.int64)
+        phys = bt[b_idx].astype(np.int64)[pos // bs] * bs + pos % bs
+        k_sel = key[phys]
+        ks_sel = ks[phys]
+        for s in range(s1):
+            t = b_idx * s1 + s
+            dot = q[t].astype(np.float32) @ k_sel.astype(np.float32).T                   # [H, n], exact
+            v = (dot * np.float32(RELU_SCALE)).astype(np.float16)
+            v = (v * qs[t][:, None]).astype(np.float16)
+            v = (v * ks_sel[None, :]).astype(np.float16)
+            v = np.maximum(v, np.float16(0.0))
+            v = (v * wt[t][:, None]).astype(np.float16)
+            acc = np.zeros(cur, dtype=np.float32)
+            for h in range(nh):
+                acc = acc + v[h].astype(np.float32)
+            rows.append(acc)
+    return rows
+
+
+def lightning_indexer_fp16_dequant_ref(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight,
+                                       act_seq_key, block_table, selected_count: int = 2048) -> torch.Tensor:
+    """Full indexer in the chained operator's arithmetic: topk_res [T, 1, selected_count] int32."""
+    t_tot = idx_query.shape[0]
+    act = [int(v) for v in (act_seq_key.tolist() if hasattr(act_seq_key, "tolist") else act_seq_key)]
+    b = len(act)
+    s1 = t_tot // b
+    rows = li_scores_fp16_dequant(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight, act, block_table, s1)
+    res = np.empty((t_tot, 1, selected_count), dtype=np.int32)
+    for b_idx in range(b):
+        for s in range(s1):
+            t = b_idx * s1 + s
+            res[t, 0] = canonical_topk(rows[t], act[b_idx] - (s1 - 1 - s), selected_count)
+    return torch.from_numpy(res)
 
 
 def canonical_topk(score: np.ndarray, eff_seq: int, k: int) -> np.ndarray:

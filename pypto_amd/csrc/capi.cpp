@@ -181,6 +181,10 @@ int li_check(const PtoLiDecodeArgs *a)
     if (a->max_blocknum_perbatch * a->block_size > pto::LI_MAX_SEQ)
         return fail(PTO_E_INVALID_ARG, "li: max_blocknum_perbatch * block_size exceeds %d", pto::LI_MAX_SEQ);
     if (a->t > (1ll << 20) || a->block_num * a->block_size > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "li: shape out of the supported range");
+    if (a->arith_variant != 0 && a->arith_variant != 1) return fail(PTO_E_INVALID_ARG, "li: arith_variant must be 0 or 1");
+    if (a->arith_variant == 1 &&
+        (a->q_scale_dtype != PTO_DT_FP16 || a->k_scale_dtype != PTO_DT_FP16 || a->weight_dtype != PTO_DT_FP16))
+        return fail(PTO_E_INVALID_ARG, "li: arith_variant 1 takes fp16 scales and weights");
     const int dts[3] = {a->q_scale_dtype, a->k_scale_dtype, a->weight_dtype};
     for (int d : dts)
         if (d != PTO_DT_FP16 && d != PTO_DT_FP32 && d != PTO_DT_BF16) return fail(PTO_E_INVALID_ARG, "li: unknown dtype code %d", d);
@@ -354,6 +358,7 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.q_dt = a->q_scale_dtype;
     p.k_dt = a->k_scale_dtype;
     p.w_dt = a->weight_dtype;
+    p.variant = a->arith_variant;
     {   // A wave pays three dependent memory latencies before its first pair, so runs are made as long
         // as still leaves every SIMD two rounds of two waves; at most 32 pairs (2048 keys) per wave.
         const long long pairs = (long long)a->t * ((p.score_stride + 63) / 64);

@@ -28,6 +28,7 @@ struct LiParams {
     int ppw;                // 64-key block pairs per wave of the score kernel, <= LI_MAX_PAIRS_PER_WAVE
     int balanced;           // score kernel sizes its runs from the sequence lengths (T <= LI_MAX_BALANCED_TOKENS)
     int score_wgs;          // its launch size in workgroups of four waves when balanced
+    int variant;            // 0: fp32 head factors applied after the ReLU; 1: fp16 scales applied before it (all tensors fp16)
 };
 
 hipError_t li_launch(const LiParams &p, hipStream_t stream);

@@ -146,6 +146,26 @@ __device__ __forceinline__ uint32_t relu_fp16_pair(const int d0, const int d1, c
     return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s16x2, packed), zero));
 }
 
+// fp16(dot / 2048) for two dots, packed, sign kept
+__device__ __forceinline__ uint32_t fp16_pair(const int d0, const int d1, const float scale)
+{
+    uint32_t packed;
+    asm("v_fma_mixlo_f16 %0, %1, %2, 0" : "=v"(packed) : "v"((float)d0), "s"(scale));
+    asm("v_fma_mixhi_f16 %0, %1, %2, 0" : "+v"(packed) : "v"((float)d1), "s"(scale));
+    return packed;
+}
+
+// two heads of one key: ((x * q_scale) * k_scale, ReLU) * weight, every product rounded to fp16
+__device__ __forceinline__ uint32_t dequant_relu_weight(const uint32_t x, const uint32_t qs, const uint32_t ks, const uint32_t w)
+{
+    typedef __attribute__((ext_vector_type(2))) short s16x2;
+    f16x2 v = __builtin_bit_cast(f16x2, x) * __builtin_bit_cast(f16x2, qs);
+    v = v * __builtin_bit_cast(f16x2, ks);
+    const s16x2 zero = {0, 0};
+    v = __builtin_bit_cast(f16x2, __builtin_elementwise_max(__builtin_bit_cast(s16x2, v), zero));
+    return __builtin_bit_cast(uint32_t, v * __builtin_bit_cast(f16x2, w));
+}
+
 constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // key rows of one staged pair of 32-key blocks
 constexpr int SC_BUF_BYTES = SC_PAIR_BYTES + 256;   // + the 64 key scales (one dword per lane)
 
@@ -169,7 +189,11 @@ constexpr int SC_BUF_BYTES = SC_PAIR_BYTES + 256;   // + the 64 key scales (one 
 // matrix instructions accumulate in ordinary vector registers and the epilogue reads them directly.
 // KDT = dtype code of the key scales: a compile-time choice keeps the scale load free of branches, so
 // it stays in flight beside the staged rows.
-template <int KDT>
+// VAR = 1: the arithmetic of the reference's chained C++ operator (LightningIndexerTopkImpl,
+// framework/src/operator/models/deepseek_v3.2_exp/lightning_indexer.cpp:149-197): fp16(dot/2048) is
+// multiplied in fp16 by the head's query scale and by the key's scale before the ReLU, then in fp16 by
+// the head's weight; the fp32 head sum (h ascending) is the score.  All three tensors are fp16 then.
+template <int KDT, int VAR = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void li_score_kernel(const LiParams p)
 {
     __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_BUF_BYTES];
@@ -296,9 +320,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             qa[1][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * LI_DIM + 16 * ks);
         }
     }
-    // per-head factors: lane l computes head l's; read back lane by lane they are wave-uniform
-    float wsc[LI_HEADS];
-    {
+    // per-head factors: lane l computes head l's; read back lane by lane they are wave-uniform.
+    // VAR = 1 keeps the fp16 query scales and weights of head pairs (2i, 2i+1) packed instead.
+    float wsc[VAR ? 1 : LI_HEADS];
+    uint32_t qs2[VAR ? LI_HEADS / 2 : 1], w2[VAR ? LI_HEADS / 2 : 1];
+    if (VAR) {
+        const uint32_t mq = reinterpret_cast<const uint32_t *>(p.q_scale)[(size_t)t * (LI_HEADS / 2) + (l & 31)];
+        const uint32_t mw = reinterpret_cast<const uint32_t *>(p.weight)[(size_t)t * (LI_HEADS / 2) + (l & 31)];
+#pragma unroll
+        for (int h = 0; h < LI_HEADS / 2; ++h) {
+            qs2[h] = (uint32_t)__builtin_amdgcn_readlane((int)mq, h);
+            w2[h] = (uint32_t)__builtin_amdgcn_readlane((int)mw, h);
+        }
+    } else {
         const float mine = w_scale_of(p, (size_t)t * LI_HEADS + l);
 #pragma unroll
         for (int h = 0; h < LI_HEADS; ++h) wsc[h] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), h));
@@ -332,6 +366,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
         __builtin_amdgcn_s_waitcnt(0xC07F);                      // lgkmcnt(0): the buffer has been read
         if (pr + 2 < npair) request_pair(pr + 2, buf);
         float ksc;
+        uint32_t ks2 = 0;                                        // the key's fp16 scale twice (VAR = 1)
         if (KDT == PTO_DT_FP32) {
             ksc = __uint_as_float(ksraw);
         } else {
@@ -341,6 +376,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             const bool odd = ((reinterpret_cast<uintptr_t>(p.k_scale) + ((size_t)(half ? rrow1 : rrow) + j) * KSZ) & 2) != 0;
             const uint16_t hbits = (uint16_t)(odd ? ksraw >> 16 : ksraw);
             ksc = KDT == PTO_DT_BF16 ? bf16_bits_to_f32(hbits) : (float)__builtin_bit_cast(_Float16, hbits);
+            ks2 = (uint32_t)hbits | ((uint32_t)hbits << 16);
         }
         i32x16 ax0, ax1, ay0, ay1;
 #pragma unroll
@@ -356,14 +392,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
         uint32_t lo[2][8], hi[2][8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const uint32_t x0 = relu_fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale), y0 = relu_fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale);
-            const uint32_t x1 = relu_fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale), y1 = relu_fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale);
+            const uint32_t x0 = VAR ? fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale) : relu_fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale);
+            const uint32_t y0 = VAR ? fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale) : relu_fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale);
+            const uint32_t x1 = VAR ? fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale) : relu_fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale);
+            const uint32_t y1 = VAR ? fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale) : relu_fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale);
             const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
             const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
             lo[0][i] = s0[0]; hi[0][i] = s0[1];
             lo[1][i] = s1[0]; hi[1][i] = s1[1];
         }
         float sum = 0.f;
+        if (VAR) {
+            const float one = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3f800000));
+#pragma unroll
+            for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t v = dequant_relu_weight(lo[o][i], qs2[8 * o + i], ks2, w2[8 * o + i]);
+                    sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
+                    sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
+                }
+            }
+#pragma unroll
+            for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t v = dequant_relu_weight(hi[o][i], qs2[16 + 8 * o + i], ks2, w2[16 + 8 * o + i]);
+                    sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
+                    sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
+                }
+            }
+            const int pos = key0 + 64 * pr + l;
+            if (pos < cur) srow[pos] = sum;
+            return;
+        }
 #pragma unroll
         for (int o = 0; o < 2; ++o) {
 #pragma unroll
@@ -953,7 +1015,8 @@ hipError_t li_launch(const LiParams &p, hipStream_t stream)
         const unsigned gx = (unsigned)((p.score_stride + 4 * p.ppw * 64 - 1) / (4 * p.ppw * 64));
         grid = dim3(gx, (unsigned)p.T);
     }
-    if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
+    if (p.variant == 1) hipLaunchKernelGGL((li_score_kernel<PTO_DT_FP16, 1>), grid, block, 0, stream, p);
+    else if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
     else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP16>, grid, block, 0, stream, p);
     else hipLaunchKernelGGL(li_score_kernel<PTO_DT_BF16>, grid, block, 0, stream, p);
     hipError_t e = hipGetLastError();

@@ -174,12 +174,18 @@ PYBIND11_MODULE(_C, m)
              std::uintptr_t block_table, std::uintptr_t topk_res, std::uintptr_t workspace, size_t workspace_bytes,
              int64_t t, int64_t b, int64_t n_heads, int64_t head_dim, int64_t block_num, int64_t block_size,
              int64_t max_blocknum_perbatch, int64_t selected_count, int q_dt, int k_dt, int w_dt,
-             std::uintptr_t stream) {
+             std::uintptr_t stream, int arith_variant) {
               PtoLiDecodeArgs a = li_args(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight, act_seq_key,
                                           block_table, topk_res, workspace, workspace_bytes, t, b, n_heads, head_dim,
                                           block_num, block_size, max_blocknum_perbatch, selected_count, q_dt, k_dt, w_dt);
+              a.arith_variant = arith_variant;
               check(pto_li_decode_launch(&a, ptr<void>(stream)));
-          });
+          },
+          py::arg("idx_query"), py::arg("idx_query_scale"), py::arg("idx_key_cache"), py::arg("idx_key_scale"),
+          py::arg("idx_weight"), py::arg("act_seq_key"), py::arg("block_table"), py::arg("topk_res"), py::arg("workspace"),
+          py::arg("workspace_bytes"), py::arg("t"), py::arg("b"), py::arg("n_heads"), py::arg("head_dim"),
+          py::arg("block_num"), py::arg("block_size"), py::arg("max_blocknum_perbatch"), py::arg("selected_count"),
+          py::arg("q_dt"), py::arg("k_dt"), py::arg("w_dt"), py::arg("stream"), py::arg("arith_variant") = 0);
 
     m.def("li_prolog_quant_workspace_bytes", [](int64_t t, int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows) {
         PtoLiPrologQuantArgs a{};

@@ -40,11 +40,18 @@ _DT = {torch.float16: 0, torch.float32: 1, torch.bfloat16: 2}
 
 def lightning_indexer_decode(idx_query, idx_query_scale, idx_key_cache, idx_key_scale, idx_weight,
                              act_seq_key, block_table, topk_res, unroll_list=None, configs=None,
-                             selected_count: int = 2048):
+                             selected_count: int = 2048, arith_variant: str = "scaled_sum"):
     """idx_query (t, 64, 128) int8; idx_query_scale (t, 64) fp16|fp32; idx_key_cache
     (block_num, block_size, 1, 128) int8; idx_key_scale (block_num, block_size, 1) fp16|fp32;
     idx_weight (t, 64) fp16|bf16|fp32; act_seq_key (b,) int32; block_table (b, max_blocks) int32;
-    topk_res (t, 1, selected_count) int32, written in place."""
+    topk_res (t, 1, selected_count) int32, written in place.
+
+    ``arith_variant`` (not part of the reference signature): ``"scaled_sum"`` is the arithmetic of this
+    operator's reference graph and golden; ``"fp16_dequant"`` is that of the reference's chained C++ operator
+    (framework/src/operator/models/deepseek_v3.2_exp/lightning_indexer.cpp:149-197; golden
+    framework/tests/st/operator/src/test_deepseek_v3.2_exp/gen_lightning_indexer.py:243-257): fp16(q.k/2048) times
+    q_scale, times k_scale (both products rounded to fp16), ReLU, times weight in fp16, fp32 head sum.  It takes
+    fp16 scales and weights only."""
     C = _native.load()
     q = as_torch(idx_query, "idx_query")
     qs = as_torch(idx_query_scale, "idx_query_scale")
@@ -90,6 +97,13 @@ def lightning_indexer_decode(idx_query, idx_query_scale, idx_key_cache, idx_key_
     if bt.shape[1] * block_size > MAX_LI_S2:
         raise ValueError(f"block_table spans more than MAX_LI_S2 = {MAX_LI_S2} positions")
 
+    if arith_variant not in ("scaled_sum", "fp16_dequant"):
+        raise ValueError(f"arith_variant: expected 'scaled_sum' or 'fp16_dequant', got {arith_variant!r}")
+    if arith_variant == "fp16_dequant" and not (qs.dtype == ks.dtype == w.dtype == torch.float16):
+        raise TypeError("arith_variant 'fp16_dequant' takes fp16 idx_query_scale, idx_key_scale and idx_weight")
+    for name, tt in (("idx_query_scale", qs), ("idx_key_scale", ks), ("idx_weight", w)):
+        if not tt.is_contiguous():
+            raise ValueError(f"{name}: must be contiguous")
     args = (t_tot, b, n_heads, d, block_num, block_size, bt.shape[1], selected_count, _DT[qs.dtype], _DT[ks.dtype],
             _DT[w.dtype])
     ws_bytes = C.li_decode_workspace_bytes(*args)
@@ -97,5 +111,6 @@ def lightning_indexer_decode(idx_query, idx_query_scale, idx_key_cache, idx_key_
     stream = torch.cuda.current_stream(dev).cuda_stream
     with torch.cuda.device(dev):
         C.li_decode_launch(q.data_ptr(), qs.data_ptr(), kc.data_ptr(), ks.data_ptr(), w.data_ptr(), act.data_ptr(),
-                           bt.data_ptr(), res.data_ptr(), ws.data_ptr(), ws_bytes, *args, stream)
+                           bt.data_ptr(), res.data_ptr(), ws.data_ptr(), ws_bytes, *args, stream,
+                           1 if arith_variant == "fp16_dequant" else 0)
     return None

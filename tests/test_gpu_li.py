@@ -127,3 +127,38 @@ def test_select_falls_back_on_degenerate_rows(c_oracle):
     ks[phys1] = ks[phys1[0]].clone()
     ks[phys1[pos1 % 4 == 1]] = ks[phys1[0]].clone() * 0.5
     assert_exact(run_op(inp), oracle(inp, c_oracle), "degenerate rows")
+
+
+def run_variant(inp):
+    dev = torch.device("cuda:0")
+    d = inp.to(dev)
+    d.topk_res.fill_(-7)
+    ret = pypto_amd.lightning_indexer_decode(*d.operator_tensors(), None, None, inp.selected_count,
+                                             arith_variant="fp16_dequant")
+    assert ret is None
+    torch.cuda.synchronize()
+    return d.topk_res.cpu()
+
+
+@pytest.mark.parametrize("b,s1,act,k", [
+    (2, 1, [4096, 3000], 2048),
+    (3, 2, [300, 129, 5], 64),
+    (1, 1, [33], 16),
+    (2, 2, [9000, 2049], 2048),
+])
+def test_fp16_dequant_variant_bit_exact(b, s1, act, k):
+    """The arithmetic of the reference's chained C++ operator (fp16 scales applied before the ReLU), against
+    its own oracle."""
+    from oracle import li_oracle as lo
+    inp = gen_indexer_inputs(b, s1, act, selected_count=k, seed=11 * b + s1 + k, variant="fp16")
+    want = lo.lightning_indexer_fp16_dequant_ref(inp.idx_query, inp.idx_query_scale, inp.idx_key_cache, inp.idx_key_scale,
+                                                 inp.idx_weight, inp.act_seq_key, inp.block_table, k)
+    assert_exact(run_variant(inp), want, f"fp16_dequant b={b} s1={s1} act={act} k={k}")
+
+
+def test_fp16_dequant_variant_refuses_other_dtypes():
+    inp = gen_indexer_inputs(1, 1, [300], selected_count=64, seed=1, variant="fp32").to(torch.device("cuda:0"))
+    with pytest.raises(TypeError):
+        pypto_amd.lightning_indexer_decode(*inp.operator_tensors(), None, None, 64, arith_variant="fp16_dequant")
+    with pytest.raises(ValueError):
+        pypto_amd.lightning_indexer_decode(*inp.operator_tensors(), None, None, 64, arith_variant="other")

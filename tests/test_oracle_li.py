@@ -216,3 +216,53 @@ def test_setwise_agreement_with_plain_torch_evaluation():
         sc = torch.matmul(w[None], x)[0] * ks[phys]
         out[b, 0] = torch.topk(sc, 512).indices.to(torch.int32)
     topk_idx_compare(out, ref, "topk_res", 5e-3, 512)
+
+
+def _fp16_rne(x: Fraction) -> float:
+    """Exact rational -> nearest fp16, ties to even; handles subnormals; overflow not needed here."""
+    if x == 0:
+        return 0.0
+    sign = -1.0 if x < 0 else 1.0
+    x = abs(x)
+    e = -14
+    while x >= Fraction(2) ** (e + 1):
+        e += 1
+    unit = Fraction(2) ** (e - 10)                    # spacing of fp16 values in [2^e, 2^(e+1)) (and below 2^-14)
+    q, r = divmod(x, unit)
+    q = int(q)
+    if 2 * r > unit or (2 * r == unit and (q & 1)):
+        q += 1
+    return sign * float(q * unit)
+
+
+def test_fp16_dequant_variant_against_exact_rationals():
+    """The chained C++ operator's rounding model: every fp16 product and the fp32 head sum restated with
+    exact rationals on a small case; and it differs from the operator's own model."""
+    inp = gen_indexer_inputs(1, 1, [40], selected_count=8, seed=5, variant="fp16", n_heads=64)
+    rows = lo.li_scores_fp16_dequant(inp.idx_query, inp.idx_query_scale, inp.idx_key_cache, inp.idx_key_scale,
+                                     inp.idx_weight, inp.act_seq, inp.block_table)
+    q = inp.idx_query[0].numpy().astype(int)
+    kc = inp.idx_key_cache.reshape(-1, 128).numpy().astype(int)
+    ks = inp.idx_key_scale.reshape(-1).numpy()
+    qs = inp.idx_query_scale[0].numpy()
+    wt = inp.idx_weight[0].numpy()
+    bt = inp.block_table[0].numpy()
+    for j in (0, 7, 39):
+        phys = int(bt[j // 128]) * 128 + j % 128
+        acc = 0.0
+        for h in range(64):
+            dot = int(np.dot(q[h], kc[phys]))
+            v = _fp16_rne(Fraction(dot, 2048))
+            v = _fp16_rne(Fraction(v) * Fraction(float(qs[h])))
+            v = _fp16_rne(Fraction(v) * Fraction(float(ks[phys])))
+            v = max(v, 0.0)
+            v = _fp16_rne(Fraction(v) * Fraction(float(wt[h])))
+            acc = _rn32(Fraction(acc) + Fraction(v))
+        assert rows[0][j] == np.float32(acc), (j, rows[0][j], acc)
+    other = lo.li_scores(inp.idx_query, inp.idx_query_scale, inp.idx_key_cache, inp.idx_key_scale, inp.idx_weight,
+                         inp.act_seq, inp.block_table)
+    assert not np.array_equal(other[0], rows[0])
+    # same ranking up to near-ties: the two models select almost the same keys
+    a = set(lo.canonical_topk(rows[0], 40, 8).tolist())
+    b = set(lo.canonical_topk(other[0], 40, 8).tolist())
+    assert len(a & b) >= 6
