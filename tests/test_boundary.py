@@ -101,3 +101,28 @@ def test_operators_refuse_cpu_tensors_loudly():
     li = gen_indexer_inputs(1, 1, [256], selected_count=64, seed=0)
     with pytest.raises(RuntimeError):
         pypto_amd.lightning_indexer_decode(*li.operator_tensors(), None, None, 64)
+
+
+def test_prolog_operators_refuse_cpu_tensors_and_unbuilt_variants():
+    import pypto_amd
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
+    kw = dict(h=128, q_lora_rank=512, n_heads=2)
+    lip = gen_indexer_prolog_inputs(1, 1, [130], seed=0, **kw)
+    outs = (torch.zeros(1, 2, 128, dtype=torch.int8), torch.zeros(1, 2, 1, dtype=torch.float16), lip.k_cache,
+            lip.k_cache_scale, torch.zeros(1, 2, dtype=torch.float16))
+    with pytest.raises(RuntimeError):
+        pypto_amd.lightning_indexer_prolog_quant(*lip.input_tensors(), *outs)
+    with pytest.raises(ValueError):
+        pypto_amd.lightning_indexer_prolog_quant(*lip.input_tensors(), *outs,
+                                                 pypto_amd.IndexerPrologQuantAttr(layerout_key="BSND"))
+    mla = gen_mla_prolog_inputs(1, 1, [130], seed=0, **kw)
+    mouts = (torch.zeros(1, 512, dtype=torch.int8), torch.zeros(1, 1), torch.zeros(1, 2, 512, dtype=torch.bfloat16),
+             torch.zeros(1, 2, 64, dtype=torch.bfloat16), mla.kv_cache, mla.kr_cache, mla.k_scale_cache)
+    with pytest.raises(RuntimeError):
+        pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "PA_BSND", None, None)
+    with pytest.raises(ValueError):
+        pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "PA_NZ", None, None)
+    args = list(mla.input_tensors())
+    args[3] = None                                       # no dequant scale: the non-quantized up-projection
+    with pytest.raises(ValueError):
+        pypto_amd.mla_prolog_quant_d(*args, *mouts, 1e-5, 1e-5, "PA_BSND", None, None)
