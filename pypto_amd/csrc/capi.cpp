@@ -204,6 +204,7 @@ int lip_check(const PtoLiPrologQuantArgs *a)
     if (a->t < 1 || a->t > (1ll << 20)) return fail(PTO_E_INVALID_ARG, "li_prolog: t must be in [1, 2^20]");
     if (a->n_heads < 1 || a->n_heads > pto::LIP_MAX_HEADS)
         return fail(PTO_E_INVALID_ARG, "li_prolog: n_heads must be in [1, %d] (got %lld)", pto::LIP_MAX_HEADS, (long long)a->n_heads);
+    static_assert(pto::LIP_MAX_QLORA == 1536, "the list below follows the kernel's instantiations");
     if (a->q_lora_rank != 512 && a->q_lora_rank != 1024 && a->q_lora_rank != 1536)
         return fail(PTO_E_INVALID_ARG, "li_prolog: q_lora_rank must be 512, 1024 or 1536 (got %lld)", (long long)a->q_lora_rank);
     const long long max_h = (long long)pto::LIP_MAX_XGROUPS * pto::LIP_XGROUP * pto::LIP_XBLOCK;

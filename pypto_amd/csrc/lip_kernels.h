@@ -7,13 +7,13 @@ namespace pto {
 
 constexpr int LIP_DIM = 128;        // channels per indexer head
 constexpr int LIP_ROPE = 64;        // leading channels that are rotated
-constexpr int LIP_KSPLIT = 4;       // workgroups that share the reduction axis of the query projection
+constexpr int LIP_KSPLIT = 4;       // workgroups that share the reduction axis of the query projection (= QPROJ_KSPLIT of the shared job code)
 constexpr int LIP_XBLOCK = 64;      // block length of the fixed-order sums over the hidden axis
 constexpr int LIP_XGROUP = 8;       // block sums per group of the second level of those sums
 constexpr int LIP_MAX_XGROUPS = 24; // groups the finishing kernel keeps in LDS: h <= 24 * 8 * 64 = 12288
 constexpr int LIP_XCOLS = 192;      // columns of one partial row: 128 key channels, then up to 64 head weights
 constexpr int LIP_MAX_HEADS = 64;
-constexpr int LIP_MAX_QLORA = 2048; // the quarter tile of w_qb (q_lora_rank/4 rows of 128 bytes) must fit in 64 KiB of LDS
+constexpr int LIP_MAX_QLORA = 1536; // a wave keeps the requests of its eighth of w_qb (q_lora_rank/8 rows) and of its token rows in flight at once (at most 63)
 
 struct LipParams {
     const uint16_t *x;           // [T, h] bf16

@@ -37,6 +37,8 @@
 namespace pto {
 namespace {
 
+static_assert(LIP_KSPLIT == QPROJ_KSPLIT, "workspace sizing and the projection job disagree");
+
 // ---------------------------------------------------------------------------------------------
 // Hidden-axis jobs: block c of 64 rows, tokens t0, t0+1.  Even jobs take wk (lane l: columns 2l,
 // 2l+1), odd jobs w_proj (lane l: column l).  The block of weights (contiguous in memory) travels to
