@@ -57,6 +57,21 @@ __device__ __forceinline__ void dequant8(const int r0, const int r1, const float
     *reinterpret_cast<u32x4 *>(dst) = out;
 }
 
+// four bytes -> four bf16 in two registers
+__device__ __forceinline__ u32x2 dequant4(const uint32_t r, const float sc)
+{
+    const float bias = -128.0f * sc;
+    const uint32_t v = r ^ 0x80808080u;
+    const float f0 = __builtin_fmaf((float)(v & 0xffu), sc, bias);
+    const float f1 = __builtin_fmaf((float)((v >> 8) & 0xffu), sc, bias);
+    const float f2 = __builtin_fmaf((float)((v >> 16) & 0xffu), sc, bias);
+    const float f3 = __builtin_fmaf((float)(v >> 24), sc, bias);
+    u32x2 out;
+    out[0] = pack_bf16x2(f0, f1);
+    out[1] = pack_bf16x2(f2, f3);
+    return out;
+}
+
 // O^T accumulators live in the accumulation registers for the whole kernel (16 blocks x 16 = all 256 of
 // them).  Inside the key loop they are touched only by the matrix product itself and by acc_scale,
 // which works on them in place through inline assembly: any plain C++ arithmetic on them makes the
@@ -100,13 +115,24 @@ constexpr float RESCALE_TAU = 8.0f;   // log2 units: the reference max moves onl
 template <int NW, bool QUANT>
 __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 {
-    // One LDS pool.  Prologue: all 32*NW query heads staged at once (PITCH elements each).  Loop: tile
-    // buffers of KT rows -- while tile n is consumed from one, tile n+1 (loaded into registers before
-    // the matrix products of tile n were issued) is de-quantised into the other; one barrier per tile.
-    // Epilogue: per-wave transposition slices.
-    constexpr int POOL_ROWS = 32 * NW > 2 * KT ? 32 * NW : 2 * KT;     // at least the two tile buffers
-    __shared__ __attribute__((aligned(16))) uint16_t pool[POOL_ROWS * PITCH];
-    __shared__ int rows_lds[SFA_MAX_CHUNK + KT];
+    // One LDS pool.  Prologue: per-wave query staging regions (QREGION bytes each).  Loop: tile
+    // buffers of KT rows -- while tile n is consumed from one, tile n+1 is de-quantised into the other
+    // (int8 cache: out of a staging ring of raw rows above the tile buffers, filled by LDS-DMA two tiles
+    // ahead); one barrier per tile.  Epilogue: per-wave transposition slices.
+    constexpr int QREGION = 20 * 1024;                                 // per wave: 16 KiB nope half + 4 KiB rope
+    constexpr int EPI_BYTES = 32 * 128 * 4;                            // per wave: 32 heads x 128 channels fp32
+    constexpr int TILES_BYTES = 2 * KT * PITCH * 2;
+    constexpr int WAVE_BYTES = NW * (QREGION > EPI_BYTES ? QREGION : EPI_BYTES);
+    constexpr int STG_NOPE = KT * DN;                                  // bytes of one staged tile: int8 rows,
+    constexpr int STG_SCALE = KT * 16;                                 // four fp32 scales per row,
+    constexpr int STG_ROPE = KT * DR * 2;                              // bf16 rope rows
+    constexpr int STG_BYTES = STG_NOPE + STG_SCALE + STG_ROPE;
+    constexpr int STG_SLOTS = 2;
+    constexpr int STG_BASE = TILES_BYTES > WAVE_BYTES ? TILES_BYTES : WAVE_BYTES;   // above everything else in the pool
+    constexpr int POOL_BYTES = STG_BASE + (QUANT ? STG_SLOTS * STG_BYTES : 0);
+    static_assert(STG_BASE % 16 == 0 && STG_BYTES % 16 == 0, "LDS-DMA destinations are 16-byte aligned");
+    __shared__ __attribute__((aligned(16))) uint16_t pool[POOL_BYTES / 2];
+    __shared__ int rows_lds[SFA_MAX_CHUNK + 3 * KT];
     uint16_t *const tile0 = pool;
     uint16_t *const tile1 = pool + KT * PITCH;
 
@@ -149,8 +175,6 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // read the last head and are never stored.  The second pass stays in flight while the row table
     // below is built.
     bf16x8 qf[KSTEPS];
-    constexpr int QREGION = 20 * 1024;                            // per wave: 16 KiB nope half + 4 KiB rope
-    static_assert(NW * QREGION <= POOL_ROWS * PITCH * 2, "Q staging must fit in the pool");
     uint8_t *const qreg = reinterpret_cast<uint8_t *>(pool) + w * QREGION;
     const uint32_t qdst = (uint32_t)(uintptr_t)(lds_byte_t *)qreg;
     const int q_head0 = hg * (32 * NW) + w * 32;
@@ -211,7 +235,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // tile" unconditionally -- no per-key and no per-tile branches.
     {
         const int n_valid = k_end - k_begin;
-        const int n_pad = n_valid > 0 ? (n_valid + KT - 1) / KT * KT + KT : 0;   // + one tile: see the loop
+        const int n_pad = n_valid > 0 ? (n_valid + 2 * KT - 1) / (2 * KT) * (2 * KT) + 2 * KT : 0;   // see the loop
         for (int i = tid; i < n_pad; i += NW * 64) {
             const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
             int blk = idx / p.bs;
@@ -231,32 +255,66 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     float m_run = -INFINITY;   // reference max, log2 domain
     float l_run = 0.f;         // running sum of exp2(s - m_run)
 
-    // gather registers of one tile: NP passes of two keys per wave (512 B int8 each), RP rope pieces
+    // Gather.  Wave w owns keys w*KT/NW .. +KT/NW of every tile.
+    //   QUANT: the rows travel cache -> LDS staging area by LDS-DMA two tiles ahead of their use (no
+    //   registers are held across the products): per tile and wave KPW/2 requests of two int8 rows
+    //   (512 B each), one of the KPW scale quadruples, KPW/8 of eight rope rows (128 B each).  The
+    //   staging ring of two tiles sits above the tile buffers; a wave
+    //   de-quantises exactly what it requested, so its own wait count is all the ordering needed.
+    //   bf16 cache: rows go straight into the tile buffer (one request per key), one tile ahead.
     constexpr int NP = KT / (2 * NW);
     constexpr int RP = (KT * (DR / 8)) / (NW * 64);
-    i32x4 raw[NP];
-    float rsc[NP];
+    constexpr int KPW = KT / NW;                                  // keys per wave and tile
+    constexpr int DMA_PER_TILE = KPW / 2 + 1 + (KPW + 7) / 8;     // requests per wave and tile
+    static_assert(2 * DMA_PER_TILE <= 48, "two tiles of requests stay outstanding");
     u32x4 rrope[RP];
 
-    // wave w gathers keys w*KT/NW .. +KT/NW of the tile; within a pass the lower half-wave takes key
-    // half*NP + i, so a lane's NP row numbers are one contiguous LDS read
-    auto issue_loads = [&](const int kt, uint16_t *buf) {
-        if (QUANT) {
-            const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW) + half * NP;
-#pragma unroll
-            for (int i = 0; i < NP; ++i) {
-                const int row = rtab[i];
-                raw[i] = *reinterpret_cast<const i32x4 *>(p.kn + (size_t)row * p.kn_pitch + 16 * col);
-                rsc[i] = *reinterpret_cast<const float *>(p.ksc + (size_t)row * p.ksc_pitch + 4 * (col >> 3));
-            }
+    // Per-lane byte offsets into the pool, kept opaque to the optimiser: every LDS access of the
+    // staged path is then "one of these registers + an immediate" instead of an address register of
+    // its own (dozens of them, at the price of spilled Q^T fragments).
+    const int wu = __builtin_amdgcn_readfirstlane(w);
+    uint32_t fetch_off = STG_BASE + w * KPW * DN + 8 * l;                          // this lane's 8 staged bytes of a key
+    uint32_t scale_off = STG_BASE + STG_NOPE + w * KPW * 16 + 4 * (l >> 4);          // their scale
+    uint32_t ropes_off = STG_BASE + STG_NOPE + STG_SCALE + 16 * (w * KPW * 8 + l);   // staged rope piece
+    uint32_t emit_off = (w * KPW * PITCH) * 2 + 16 * l;                              // the 8 de-quantised channels
+    uint32_t ropee_off = ((w * KPW + (l >> 3)) * PITCH + DN + 8 * (l & 7)) * 2;      // rope piece in the tile
+    if (QUANT) asm volatile("" : "+v"(fetch_off), "+v"(scale_off), "+v"(ropes_off), "+v"(emit_off), "+v"(ropee_off));
+    uint8_t *const pool_b = reinterpret_cast<uint8_t *>(pool);
+
+    // Request k of a tile (QUANT only): k < KPW/2 two int8 rows, k == KPW/2 the scale quadruples, then
+    // eight rope rows each.  stage_row reads the cache row number a lane needs for request k,
+    // stage_request issues it.
+    auto stage_row = [&](const int kt, const int k) {
+        const int *rtab = rows_lds + (kt - k_begin) + wu * KPW;
+        if (k < KPW / 2) return rtab[2 * k + half];
+        if (k == KPW / 2) return rtab[l & (KPW - 1)];
+        return rtab[8 * (k - KPW / 2 - 1) + (l >> 3)];
+    };
+    auto stage_request = [&](const int slot, const int k, const int row) {
+        const uint32_t dst = (uint32_t)(uintptr_t)(lds_byte_t *)pool_b + STG_BASE + slot * STG_BYTES;
+        if (k < KPW / 2) {
+            dma16(p.kn + (size_t)row * p.kn_pitch + 16 * col, dst + (wu * KPW + 2 * k) * DN);
+        } else if (k == KPW / 2) {
+            if (l < KPW) dma16(p.ksc + (size_t)row * p.ksc_pitch, dst + STG_NOPE + wu * KPW * 16);
         } else {
-            // one request per key: the 64 lanes' 16-byte pieces are the 1024 bytes of the row, in order
-            const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW);
-#pragma unroll
-            for (int i = 0; i < KT / NW; ++i)
-                dma16(p.kn + (size_t)rtab[i] * p.kn_pitch + 16 * l,
-                      (uint32_t)(uintptr_t)(lds_byte_t *)(buf + (w * (KT / NW) + i) * PITCH));
+            dma16(p.kr + (size_t)row * p.kr_pitch + 16 * (l & 7),
+                  dst + STG_NOPE + STG_SCALE + (wu * KPW + 8 * (k - KPW / 2 - 1)) * (DR * 2));
         }
+    };
+    auto stage_tile = [&](const int kt, const int slot) {          // a whole tile at once: the prologue
+        int rows[DMA_PER_TILE];
+#pragma unroll
+        for (int k = 0; k < DMA_PER_TILE; ++k) rows[k] = stage_row(kt, k);
+#pragma unroll
+        for (int k = 0; k < DMA_PER_TILE; ++k) stage_request(slot, k, rows[k]);
+    };
+    auto issue_loads = [&](const int kt, uint16_t *buf) {          // bf16 cache only
+        // one request per key: the 64 lanes' 16-byte pieces are the 1024 bytes of the row, in order
+        const int *rtab = rows_lds + (kt - k_begin) + w * (KT / NW);
+#pragma unroll
+        for (int i = 0; i < KT / NW; ++i)
+            dma16(p.kn + (size_t)rtab[i] * p.kn_pitch + 16 * l,
+                  (uint32_t)(uintptr_t)(lds_byte_t *)(buf + (w * (KT / NW) + i) * PITCH));
 #pragma unroll
         for (int i = 0; i < RP; ++i) {
             const int e = tid + i * NW * 64;
@@ -264,21 +322,54 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * p.kr_pitch + 16 * (e & 7));
         }
     };
-    // de-quantise and store one eighth of the gathered tile (piece 0 also stores the rope part)
-    auto store_piece = [&](uint16_t *buf, const int piece) {
-        static_assert(NP * 2 % 8 == 0 || NP * 2 == 8 || true, "");
-        constexpr int HALVES = 2 * NP;                 // 16-byte LDS stores of this lane per tile
-        constexpr int PER = (HALVES + 7) / 8;          // ... per piece
+    // De-quantisation of a staged tile, one eighth ("piece") at a time: fetch_piece reads the staged
+    // bytes into a few registers, emit_half de-quantises one half of them into the tile buffer.  The loop
+    // spreads the sixteen halves over its seventeen groups of four matrix products, each piece fetched
+    // one group before its first half is used, so that neither the LDS latency nor the vector
+    // instructions (about three per product) hold the matrix pipeline up.
+    constexpr int PER = (KPW + 7) / 8;             // keys of this wave per piece
+    u32x2 praw[2][QUANT ? PER : 1], plow[QUANT ? PER : 1];
+    float psc[2][QUANT ? PER : 1];
+    auto fetch_piece = [&](const int piece, const int slot) {
 #pragma unroll
         for (int q = 0; q < PER; ++q) {
-            const int hidx = piece * PER + q;
-            if (QUANT && hidx < HALVES) {
-                const int i = hidx >> 1, hh = hidx & 1;
-                const int kl = w * (KT / NW) + half * NP + i;
-                dequant8(raw[i][2 * hh], raw[i][2 * hh + 1], rsc[i], buf + kl * PITCH + 16 * col + 8 * hh);
+            const int i = piece * PER + q;         // key of this wave: a wave instruction covers its 512 bytes
+            if (i < KPW) {
+                praw[piece & 1][q] = *reinterpret_cast<const u32x2 *>(pool_b + fetch_off + (slot * STG_BYTES + i * DN));
+                psc[piece & 1][q] = *reinterpret_cast<const float *>(pool_b + scale_off + (slot * STG_BYTES + i * 16));
             }
         }
-        if (piece == 0) {
+    };
+    // tile = 0 or 1: which of the two tile buffers.  Half 0 converts the lower four bytes, half 1 the upper
+    // four and stores the eight channels (the wave's 64 lanes: 1024 contiguous bytes of the key's row).
+    auto emit_half = [&](const int tile, const int piece, const int hf) {
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int i = piece * PER + q;
+            if (i < KPW) {
+                const u32x2 c = dequant4(praw[piece & 1][q][hf], psc[piece & 1][q]);
+                if (hf == 0) {
+                    plow[q] = c;
+                } else {
+                    u32x4 v;
+                    v[0] = plow[q][0], v[1] = plow[q][1], v[2] = c[0], v[3] = c[1];
+                    *reinterpret_cast<u32x4 *>(pool_b + emit_off + (tile * KT * PITCH * 2 + i * PITCH * 2)) = v;
+                }
+            }
+        }
+    };
+    auto fetch_rope = [&](const int slot) {
+#pragma unroll
+        for (int i = 0; i < RP; ++i)
+            rrope[i] = *reinterpret_cast<const u32x4 *>(pool_b + ropes_off + (slot * STG_BYTES + i * 1024));
+    };
+    auto emit_rope = [&](const int tile) {
+        if (QUANT) {
+#pragma unroll
+            for (int i = 0; i < RP; ++i)
+                *reinterpret_cast<u32x4 *>(pool_b + ropee_off + (tile * KT * PITCH * 2 + i * 8 * PITCH * 2)) = rrope[i];
+        } else {
+            uint16_t *buf = tile ? tile1 : tile0;
 #pragma unroll
             for (int i = 0; i < RP; ++i) {
                 const int e = tid + i * NW * 64;
@@ -286,29 +377,84 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
         }
     };
-    auto store_tile = [&](uint16_t *buf) {
+    // what group u = 0..16 of a tile's products does for the next tile, before and after its products
+    // ... and for the tile after the next: its requests, REQ_PER_GROUP in each of the groups 1.., the cache
+    // row numbers read one group earlier (issued all at once the requests of the four waves queue up at
+    // the address unit for several hundred cycles; spread out they pass under the products)
+    constexpr int REQ_PER_GROUP = (DMA_PER_TILE + 15) / 16;
+    int srow[REQ_PER_GROUP];
+    auto group_pre = [&](const int u, const int slot, const int kt2, const int slot2) {
+        if (!QUANT) return;
+        if (u % 2 == 0 && u / 2 < 8) fetch_piece(u / 2, slot);
+        if (u == 15) fetch_rope(slot);
 #pragma unroll
-        for (int piece = 0; piece < 8; ++piece) store_piece(buf, piece);
+        for (int j = 0; j < REQ_PER_GROUP; ++j) {
+            const int k = (u - 1) * REQ_PER_GROUP + j;
+            if (u >= 1 && k < DMA_PER_TILE) stage_request(slot2, k, srow[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < REQ_PER_GROUP; ++j) {
+            const int k = u * REQ_PER_GROUP + j;
+            if (k < DMA_PER_TILE) srow[j] = stage_row(kt2, k);
+        }
+    };
+    auto group_post = [&](const int u, const int tile) {
+        if (QUANT) {
+            if (u >= 1) emit_half(tile, (u - 1) / 2, (u - 1) % 2);
+            if (u == 16) emit_rope(tile);
+        } else if (u == KSTEPS / 4) {
+            emit_rope(tile);
+        }
+    };
+    auto store_tile = [&](const int tile, const int slot) {        // the first tile: nothing to hide behind
+        if (QUANT) {
+#pragma unroll
+            for (int piece = 0; piece < 8; ++piece) {
+                fetch_piece(piece, slot);
+                emit_half(tile, piece, 0);
+                emit_half(tile, piece, 1);
+            }
+            fetch_rope(slot);
+        }
+        emit_rope(tile);
     };
 
     collect_q(1);
     __syncthreads();                       // row table complete, pool free again
     if (k_begin < k_end) {
-        issue_loads(k_begin, tile0);
-        store_tile(tile0);
+        if (QUANT) {
+            stage_tile(k_begin, 0);
+            stage_tile(k_begin + KT, 1);
+            __builtin_amdgcn_s_waitcnt((DMA_PER_TILE & 15) | ((DMA_PER_TILE >> 4) << 14) | 0x0F70);   // the first tile has landed
+            asm volatile("" ::: "memory");
+        } else {
+            issue_loads(k_begin, tile0);
+        }
+        store_tile(0, 0);
     }
     if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);     // this wave's direct requests into the tile have landed
     __syncthreads();
     // All global loads issued so far (Q^T fragments, first tile) are complete from here on, so that
-    // inside the loop the only outstanding vector-memory operations are the next tile's gather and
-    // the compiler's wait counts do not serialise it with the matrix products.
-    __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0), expcnt and lgkmcnt unconstrained
+    // inside the loop the only outstanding vector-memory operations are the gathers of later tiles and
+    // the compiler's wait counts do not serialise them with the matrix products.
+    if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0), expcnt and lgkmcnt unconstrained
 
-    int it = 0;
-    for (int kt = k_begin; kt < k_end; kt += KT, ++it) {
+    // One tile.  For the int8 cache the parity of the tile number is a compile-time constant (the loop
+    // below runs two tiles per trip), so every LDS address in here is a per-lane base plus an immediate
+    // offset.
+    auto tile_step = [&](auto parity, const int kt) __attribute__((always_inline)) {
+        const int it = parity;
         const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
         uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
-        issue_loads(kt + KT, nxt_tile);          // next tile (or the padding tile): in flight during the products
+        // next tile (or a padding tile) of the bf16 cache, the tile after it of the int8 cache: in flight
+        // during the products
+        if (QUANT) {
+            // the next tile's requests went out during the previous tile's products: staged by now
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            asm volatile("" ::: "memory");
+        } else {
+            issue_loads(kt + KT, nxt_tile);
+        }
 
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
@@ -321,6 +467,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             for (int e = 0; e < 4; ++e) fa[0][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * e);
 #pragma unroll
             for (int g = 0; g < KSTEPS / 4; ++g) {
+                group_pre(g, (it + 1) & 1, kt + 2 * KT, it & 1);
                 if (g + 1 < KSTEPS / 4) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
@@ -329,6 +476,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[g & 1][e], qf[4 * g + e], s, 0, 0, 0);
+                group_post(g, (it + 1) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -387,6 +535,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
+                group_pre(KSTEPS / 4 + g, (it + 1) & 1, kt + 2 * KT, it & 1);
                 if (g + 1 < 8) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -402,14 +551,25 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                     const s16x8 a = __builtin_shufflevector(va[g & 1][e][0], va[g & 1][e][1], 0, 1, 2, 3, 4, 5, 6, 7);
                     acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf[m >> 4]);
                 }
-                // one eighth of the next tile's de-quantisation rides in the shadow of these products
-                store_piece(nxt_tile, g);
+                // a sixteenth of the next tile's de-quantisation rides in the shadow of these products
+                group_post(KSTEPS / 4 + g, (it + 1) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's direct requests into the next tile have landed
         __syncthreads();
+    };
+    if constexpr (QUANT) {
+        // an odd number of tiles is rounded up: the extra tile holds padding rows only, all of them masked
+        for (int kt = k_begin; kt < k_end; kt += 2 * KT) {
+            tile_step(std::integral_constant<int, 0>{}, kt);
+            tile_step(std::integral_constant<int, 1>{}, kt + KT);
+        }
+    } else {
+        int it = 0;
+        for (int kt = k_begin; kt < k_end; kt += KT, ++it) tile_step(it & 1, kt);
     }
+    if (QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);      // the padding tiles' requests have landed: the pool is quiet
 
     // ---- epilogue.  Lane (head, half) holds value channels 32*dvb + 8*(r/4) + 4*half + r%4 of its head;
     // written from there each store instruction would touch 32 rows with 32 bytes each.  Each wave
