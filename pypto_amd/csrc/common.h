@@ -65,4 +65,13 @@ __device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
 }
 
+// four bytes per lane: lane i's dword at gaddr lands at lds_dst + 4*i
+__device__ __forceinline__ void dma4(const void *gaddr, const uint32_t lds_dst)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
+}
+// s_waitcnt immediate for "at most n vector-memory operations outstanding" (the other counters unconstrained)
+constexpr int vmcnt_imm(const int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
 }  // namespace pto

@@ -211,8 +211,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
         }
     };
-    auto collect_q = [&](const int pass) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);                       // vmcnt(0): the pass has landed
+    // pending: the number of younger requests of this wave that may still be in flight
+    auto collect_q = [&](const int pass, auto pending) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(decltype(pending)::value));   // the pass has landed
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int ks = 0; ks < 16; ++ks)
@@ -225,24 +226,65 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xC07F);                       // lgkmcnt(0): the slice may be overwritten
     };
-    request_q(0);
-    collect_q(0);
-    request_q(1);
-
-    // logical position -> physical cache row for this split's keys.  The table is padded to a whole
-    // number of tiles plus one with the row of the split's first key: keys past k_end are then loaded
-    // like any other (finite data) and masked out of the softmax, and the loop can prefetch "the next
-    // tile" unconditionally -- no per-key and no per-tile branches.
-    {
-        const int n_valid = k_end - k_begin;
-        const int n_pad = n_valid > 0 ? (n_valid + 2 * KT - 1) / (2 * KT) * (2 * KT) + 2 * KT : 0;   // see the loop
+    // logical position -> physical cache row for this split's keys.  The table is padded to an even
+    // number of tiles plus two with the row of the split's first key: keys past k_end are then loaded
+    // like any other (finite data) and masked out of the softmax, and the loop can prefetch two tiles
+    // ahead unconditionally -- no per-key and no per-tile branches.
+    //
+    // The translation is a chain of two dependent loads (selected position, then its page in the block
+    // table) ahead of the gather itself.  When the table fits two entries per thread both loads travel
+    // as LDS-DMA requests between the Q^T passes, waited for by count, so that the chain runs beside
+    // the Q^T staging instead of after it; each lane handles the entries it requested itself.
+    const int n_valid = k_end - k_begin;
+    const int n_pad = n_valid > 0 ? (n_valid + 2 * KT - 1) / (2 * KT) * (2 * KT) + 2 * KT : 0;
+    constexpr int FAST_ENTRIES = 2 * NW * 64;
+    static_assert(2 * FAST_ENTRIES <= SFA_MAX_CHUNK + 3 * KT, "positions and pages of the short table share its memory");
+    const bool fast = n_valid > 0 && n_pad <= FAST_ENTRIES;                    // uniform
+    const int wave_first = __builtin_amdgcn_readfirstlane(w) * 64;
+    auto row_of = [&](const int idx, const int page) {
+        long long row = (long long)page * p.bs + (idx - (idx / p.bs) * p.bs);
+        row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
+        return (int)row;
+    };
+    auto block_of = [&](const int idx) {
+        const int blk = idx / p.bs;
+        return blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
+    };
+    if (fast) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = tid + j * NW * 64;
+            dma4(p.topk_idx + (size_t)t * p.topk + k_begin + (i < n_valid ? i : 0),
+                 (uint32_t)(uintptr_t)(lds_byte_t *)(rows_lds + j * NW * 64 + wave_first));
+        }
+    }
+    request_q(0);                                                             // 16 requests
+    if (fast) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(16));                            // the positions have landed
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = tid + j * NW * 64;
+            dma4(p.bt + (size_t)b * p.maxblk + block_of(rows_lds[i]),
+                 (uint32_t)(uintptr_t)(lds_byte_t *)(rows_lds + FAST_ENTRIES + j * NW * 64 + wave_first));
+        }
+        collect_q(0, std::integral_constant<int, 2>{});
+    } else {
+        collect_q(0, std::integral_constant<int, 0>{});
+    }
+    request_q(1);                                                             // 20 requests
+    if (fast) {
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(20));                            // the pages have landed
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = tid + j * NW * 64;
+            rows_lds[i] = row_of(rows_lds[i], rows_lds[FAST_ENTRIES + i]);
+        }
+    } else {
         for (int i = tid; i < n_pad; i += NW * 64) {
             const int idx = p.topk_idx[(size_t)t * p.topk + k_begin + (i < n_valid ? i : 0)];
-            int blk = idx / p.bs;
-            blk = blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
-            long long row = (long long)p.bt[(size_t)b * p.maxblk + blk] * p.bs + (idx - (idx / p.bs) * p.bs);
-            row = row < 0 ? 0 : (row >= p.kv_rows ? p.kv_rows - 1 : row);
-            rows_lds[i] = (int)row;
+            rows_lds[i] = row_of(idx, p.bt[(size_t)b * p.maxblk + block_of(idx)]);
         }
     }
 
@@ -419,13 +461,20 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         emit_rope(tile);
     };
 
-    collect_q(1);
-    __syncthreads();                       // row table complete, pool free again
-    if (k_begin < k_end) {
+    __syncthreads();                       // row table complete
+    if (QUANT && n_valid > 0) {
+        // the staging ring lies above the Q^T staging: the first two tiles set out before the second
+        // Q^T pass is collected
+        stage_tile(k_begin, 0);
+        stage_tile(k_begin + KT, 1);
+        collect_q(1, std::integral_constant<int, 2 * DMA_PER_TILE>{});
+    } else {
+        collect_q(1, std::integral_constant<int, 0>{});
+    }
+    __syncthreads();                       // every wave holds its Q^T fragments: the tile buffers are free
+    if (n_valid > 0) {
         if (QUANT) {
-            stage_tile(k_begin, 0);
-            stage_tile(k_begin + KT, 1);
-            __builtin_amdgcn_s_waitcnt((DMA_PER_TILE & 15) | ((DMA_PER_TILE >> 4) << 14) | 0x0F70);   // the first tile has landed
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(DMA_PER_TILE));              // the first tile has landed
             asm volatile("" ::: "memory");
         } else {
             issue_loads(k_begin, tile0);
