@@ -82,6 +82,20 @@ __device__ __forceinline__ void acc_mfma(f32x16 &acc, const bf16x8 a, const bf16
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
 
+// S^T accumulator: kept in architectural registers by construction.  Left to the compiler it shares the
+// first sixteen accumulation registers with the first O^T block, which is then copied out and back
+// around every tile.  First product of a chain starts from zero; the chain is dependent products on one
+// destination (no wait states needed between them); s_chain_done pads the matrix-write -> vector-read slot.
+__device__ __forceinline__ void s_mfma_first(f32x16 &s, const bf16x8 a, const bf16x8 b)
+{
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void s_mfma(f32x16 &s, const bf16x8 a, const bf16x8 b)
+{
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void s_chain_done(f32x16 &s) { asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s)); }
+
 // acc *= alpha, one register at a time through a single architectural temporary (rare path)
 __device__ __forceinline__ void acc_scale(f32x16 &acc, const float alpha)
 {
@@ -507,8 +521,6 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
         {
             const uint16_t *arow = cur_tile + col * PITCH + 8 * half;
             bf16x8 fa[2][4];
@@ -523,12 +535,15 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                         fa[(g + 1) & 1][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * (4 * (g + 1) + e));
                 }
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[g & 1][e], qf[4 * g + e], s, 0, 0, 0);
+                for (int e = 0; e < 4; ++e) {
+                    if (g == 0 && e == 0) s_mfma_first(s, fa[0][0], qf[0]);
+                    else s_mfma(s, fa[g & 1][e], qf[4 * g + e]);
+                }
                 group_post(g, (it + 1) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        s_chain_done(s);
 
         // ---- online softmax; lane (head, half) holds keys kt + 8*(r/4) + 4*half + r%4
         float mx = -INFINITY;
@@ -549,14 +564,14 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         const float m_new = upd ? mx : m_run;
         const float alpha = upd ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
         const bool rescale = upd && l_run > 0.f;            // nothing accumulated yet: nothing to rescale
+        // The exponentials of the first sixteen keys are taken here; those of the other sixteen (needed by
+        // the second half of the PV products only) ride in the shadow of the first PV groups.
         float lsum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 8; ++r) {
             s[r] = __builtin_amdgcn_exp2f(s[r] - m_new);      // v_exp_f32; exp2(-inf) = 0
             lsum += s[r];
         }
-        lsum += __shfl_xor(lsum, 32);
-        l_run = l_run * alpha + lsum;
         m_run = m_new;
         if (__any(rescale)) {
             mfma_to_valu_fence();
@@ -564,13 +579,25 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             valu_to_mfma_fence();
         }
         bf16x8 pf[2];
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
+        auto pack_p = [&](const int kk) {
             u32x4 pk;
 #pragma unroll
             for (int e = 0; e < 4; ++e) pk[e] = pack_bf16x2(s[8 * kk + 2 * e], s[8 * kk + 2 * e + 1]);
             pf[kk] = __builtin_bit_cast(bf16x8, pk);
-        }
+        };
+        pack_p(0);
+        auto softmax_tail = [&](const int part) {
+#pragma unroll
+            for (int r = 8 + 4 * part; r < 12 + 4 * part; ++r) {
+                s[r] = __builtin_amdgcn_exp2f(s[r] - m_new);
+                lsum += s[r];
+            }
+            if (part == 1) {
+                pack_p(1);
+                lsum += __shfl_xor(lsum, 32);
+                l_run = l_run * alpha + lsum;
+            }
+        };
 
         // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead;
         // interleaved with the de-quantisation of the next tile into the other buffer
@@ -600,6 +627,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                     const s16x8 a = __builtin_shufflevector(va[g & 1][e][0], va[g & 1][e][1], 0, 1, 2, 3, 4, 5, 6, 7);
                     acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf[m >> 4]);
                 }
+                if (g < 2) softmax_tail(g);
                 // a sixteenth of the next tile's de-quantisation rides in the shadow of these products
                 group_post(KSTEPS / 4 + g, (it + 1) & 1);
                 __builtin_amdgcn_sched_barrier(0);
