@@ -649,21 +649,19 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     if (QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);      // the padding tiles' requests have landed: the pool is quiet
 
     // ---- epilogue.  Lane (head, half) holds value channels 32*dvb + 8*(r/4) + 4*half + r%4 of its head;
-    // written from there each store instruction would touch 32 rows with 32 bytes each.  Each wave
+    // written from there each store instruction would touch 32 rows with 8 bytes each.  Each wave
     // instead transposes 128 channels at a time through its own slice of the (now idle) tile
-    // memory, so that 32 lanes write 512 contiguous bytes of one head (256 for the bf16 result).
+    // memory, so that 16 lanes write 256 contiguous bytes of one head.
     mfma_to_valu_fence();
     {
-        // staging slice of this wave: 32 heads x 128 channels fp32, 16-byte chunk c of head h stored at
-        // chunk c ^ (h & 7): both the column-wise writes and the row-wise reads are bank-conflict free.
-        // The accumulators go to LDS as they are (the 1/l factor is applied on the way out, from a
-        // small per-head table), and the way out is a rolled loop: the straight-line part of the
-        // epilogue is one LDS store per four accumulator registers.
-        float *stage = reinterpret_cast<float *>(pool) + w * (32 * 128);
-        float *inv_tab = reinterpret_cast<float *>(rows_lds) + w * 32;      // the row table is dead by now
+        // staging slice of this wave: 32 heads x 128 channels of 16 bits, already scaled by 1/l (a lane's
+        // registers all belong to its own head) and converted, in 8-byte chunks of four channels; chunk c
+        // of head h is stored at chunk c ^ h: the column-wise writes (32 heads, one chunk) and the
+        // row-wise reads (two heads, 16 even or odd chunks each) both touch every bank once.
+        uint8_t *stage = reinterpret_cast<uint8_t *>(pool) + w * (32 * 256);
         const int head_base = hg * (32 * NW) + w * 32;
         const size_t prow_base = ((size_t)t * p.nsplit + sp) * p.NQ;
-        if (half == 0) inv_tab[col] = l_run > 0.f ? 1.0f / l_run : 0.f;
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         // FINAL: bf16 result rows; otherwise fp16 partial of a key split (O / l of the split, merged by
         // the combine kernel with weights l * 2^(m - m_max); O / l is a convex combination of
         // de-quantised V rows, so it stays finite in fp16 as long as |int8 * scale| < 65504).
@@ -672,8 +670,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         auto drain = [&](auto final_tag, auto all_tag) {
             constexpr bool FINAL = decltype(final_tag)::value;
             constexpr bool ALL = decltype(all_tag)::value;
-            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + half) * DN + 4 * col
-                                   : p.part_o + (prow_base + head_base + half) * DN + 4 * col;
+            const int hsub = l >> 4, j = l & 15;          // on the way out: head 4*e + hsub, channels 8*j .. 8*j+7
+            uint16_t *dst0 = FINAL ? p.out + ((size_t)t * p.NQ + head_base + hsub) * DN + 8 * j
+                                   : p.part_o + (prow_base + head_base + hsub) * DN + 8 * j;
 #pragma unroll
             for (int gq = 0; gq < DVB / 4; ++gq) {
 #pragma unroll
@@ -681,29 +680,21 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 #pragma unroll
                     for (int q4 = 0; q4 < 4; ++q4) {
                         const f32x16 &acc = o[4 * gq + b4];
-                        const f32x4 v = {acc[4 * q4], acc[4 * q4 + 1], acc[4 * q4 + 2], acc[4 * q4 + 3]};
-                        *reinterpret_cast<f32x4 *>(stage + col * 128 + 4 * ((8 * b4 + 2 * q4 + half) ^ (col & 7))) = v;
-                    }
-#pragma unroll 1
-                for (int pq = 0; pq < 2; ++pq) {
-                    f32x4 rv[8];
-                    float iv[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int hl = 2 * (8 * pq + e) + half;
-                        rv[e] = *reinterpret_cast<const f32x4 *>(stage + hl * 128 + 4 * (col ^ (hl & 7)));
-                        iv[e] = inv_tab[hl];
-                    }
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int hl = 2 * (8 * pq + e) + half;
-                        const f32x4 v = rv[e] * iv[e];
+                        const float v0 = acc[4 * q4] * inv, v1 = acc[4 * q4 + 1] * inv;
+                        const float v2 = acc[4 * q4 + 2] * inv, v3 = acc[4 * q4 + 3] * inv;
                         u32x2 pk;
-                        pk[0] = FINAL ? pack_bf16x2(v[0], v[1]) : pack_f16x2(v[0], v[1]);
-                        pk[1] = FINAL ? pack_bf16x2(v[2], v[3]) : pack_f16x2(v[2], v[3]);
-                        if (ALL || head_base + hl < p.NQ)
-                            *reinterpret_cast<u32x2 *>(dst0 + (size_t)(hl - half) * DN + 128 * gq) = pk;
+                        pk[0] = FINAL ? pack_bf16x2(v0, v1) : pack_f16x2(v0, v1);
+                        pk[1] = FINAL ? pack_bf16x2(v2, v3) : pack_f16x2(v2, v3);
+                        *reinterpret_cast<u32x2 *>(stage + col * 256 + 8 * ((8 * b4 + 2 * q4 + half) ^ col)) = pk;
                     }
+#pragma unroll 2
+                for (int e = 0; e < 8; ++e) {
+                    const int hl = 4 * e + hsub;
+                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(stage + hl * 256 + 8 * ((2 * j) ^ hl));
+                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(stage + hl * 256 + 8 * ((2 * j + 1) ^ hl));
+                    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+                    if (ALL || head_base + hl < p.NQ)
+                        *reinterpret_cast<u32x4 *>(dst0 + (size_t)(4 * e) * DN + 128 * gq) = v;
                 }
             }
         };
