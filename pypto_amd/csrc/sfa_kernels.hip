@@ -462,15 +462,28 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             emit_rope(tile);
         }
     };
-    auto store_tile = [&](const int tile, const int slot) {        // the first tile: nothing to hide behind
+    // the first tile has nothing to hide behind: its staged bytes are fetched in batches of eight keys,
+    // so that the LDS round trips overlap instead of following one another
+    auto store_tile = [&](const int tile, const int slot) {
         if (QUANT) {
-#pragma unroll
-            for (int piece = 0; piece < 8; ++piece) {
-                fetch_piece(piece, slot);
-                emit_half(tile, piece, 0);
-                emit_half(tile, piece, 1);
-            }
             fetch_rope(slot);
+            constexpr int BATCH = KPW < 8 ? KPW : 8;
+#pragma unroll
+            for (int i0 = 0; i0 < KPW; i0 += BATCH) {
+                u32x2 r[BATCH];
+                float sc[BATCH];
+#pragma unroll
+                for (int i = 0; i < BATCH; ++i) {
+                    r[i] = *reinterpret_cast<const u32x2 *>(pool_b + fetch_off + (slot * STG_BYTES + (i0 + i) * DN));
+                    sc[i] = *reinterpret_cast<const float *>(pool_b + scale_off + (slot * STG_BYTES + (i0 + i) * 16));
+                }
+#pragma unroll
+                for (int i = 0; i < BATCH; ++i) {
+                    const u32x2 lo = dequant4(r[i][0], sc[i]), hi = dequant4(r[i][1], sc[i]);
+                    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+                    *reinterpret_cast<u32x4 *>(pool_b + emit_off + (tile * KT * PITCH * 2 + (i0 + i) * PITCH * 2)) = v;
+                }
+            }
         }
         emit_rope(tile);
     };
