@@ -122,6 +122,14 @@ template <int N> struct AccLoop<N, N> {
 __device__ __forceinline__ void mfma_to_valu_fence() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 __device__ __forceinline__ void valu_to_mfma_fence() { asm volatile("s_nop 4" ::: "memory"); }
 
+// both half-waves' values of x, in every lane: one register-to-register exchange (no LDS round trip)
+__device__ __forceinline__ void both_halves(const float x, float &lo, float &hi)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    lo = __uint_as_float(r[0]);
+    hi = __uint_as_float(r[1]);
+}
+
 constexpr float RESCALE_TAU = 8.0f;   // log2 units: the reference max moves only when exceeded by 2^8
 
 // QUANT: the latent part of a cache row is int8 with four fp32 scales and is de-quantised on the way into
@@ -570,7 +578,11 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             s[r] *= p.scale_log2;
             mx = fmaxf(mx, s[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        {
+            float lo, hi;
+            both_halves(mx, lo, hi);
+            mx = fmaxf(lo, hi);
+        }
         // The reference max follows the true max lazily: probabilities may reach 2^RESCALE_TAU, which
         // fp32 sums and bf16 P hold without loss, and the accumulators are rescaled only on a jump.
         const bool upd = mx > m_run + RESCALE_TAU;          // always true on the first tile (m_run = -inf)
@@ -607,7 +619,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
             if (part == 1) {
                 pack_p(1);
-                lsum += __shfl_xor(lsum, 32);
+                float lo, hi;
+                both_halves(lsum, lo, hi);
+                lsum = lo + hi;
                 l_run = l_run * alpha + lsum;
             }
         };
