@@ -187,6 +187,40 @@ def mla_prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=10, replays=10):
             "hbm_frac": byt / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
 
 
+def other_shapes_leg(torch, pypto_amd, dev):
+    """configs[3] and configs[4] through the same operators (parity of both is a GPU test): step time and the
+    fraction of the dense bf16 peak their algorithmic flops reach.  Row (b, s) attends
+    min(max(act[b] - S1 + 1 + s, 0), 2048) keys."""
+    from pypto_amd.synthetic import config_lengths, gen_sfa_inputs
+    res = []
+    for name, b, s1, lengths, entry, steps in (
+            ("configs[3]: B=64 S_q=2 KV 4096-32768", 64, 2, config_lengths(3, seed=3), "d", 50),
+            ("configs[4]: B=1 S_q=4096 KV 4096 (row t sees min(t+1, 2048) keys)", 1, 4096, config_lengths(4), "p", 10)):
+        inp = gen_sfa_inputs(b, s1, 128, lengths, topk=2048, seed=5).to(dev)
+        out = torch.empty([b, s1, 128, 512], dtype=torch.bfloat16, device=dev)
+        fn = pypto_amd.sparse_flash_attention_quant_d if entry == "d" else pypto_amd.sparse_flash_attention_quant_p
+
+        def step():
+            fn(inp.query_nope, inp.query_rope, inp.key_nope_2d, inp.key_rope_2d, inp.k_nope_scales, inp.topk_indices,
+               inp.block_table, inp.kv_act_seqs, out, 128, 1, inp.softmax_scale, 2048, 128, inp.max_blocknum_perbatch, None)
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        keys = sum(min(max(int(lengths[bi]) - s1 + 1 + si, 0), 2048) for bi in range(b) for si in range(s1))
+        flops = 2.0 * 128 * keys * 1088
+        res.append({"workload": name, "us_per_step": ms * 1e3, "tokens_per_s": b * s1 / (ms * 1e-3),
+                    "tflops": flops / (ms * 1e-3) / 1e12, "mfma_frac": flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS})
+        del inp, out
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -197,6 +231,9 @@ def main():
                     help="for rocprofv3 --pmc: a few attention steps plus one device copy of COPY_MIB MiB "
                          "(the calibration kernel of the counters), no timing, no JSON line")
     ap.add_argument("--seed", type=int, default=2)
+    ap.add_argument("--other-shapes", action="store_true",
+                    help="also time configs[3] (B=64, two query tokens) and configs[4] (4096-token prefill chunk) "
+                         "and add them to the JSON line as 'other_shapes'")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -361,6 +398,8 @@ def main():
         "mla_prolog": mla_prolog,
         "cpu_baseline": cpu,
     }
+    if args.other_shapes:
+        line["other_shapes"] = other_shapes_leg(torch, pypto_amd, dev)
     print(json.dumps(line))
 
 

@@ -598,7 +598,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             lsum += s[r];
         }
         m_run = m_new;
-        if (__any(rescale)) {
+        if (__builtin_expect(__any(rescale), 0)) {               // rare: laid out away from the loop body
             mfma_to_valu_fence();
             AccLoop<0, DVB>::scale(o, alpha);
             valu_to_mfma_fence();
