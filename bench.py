@@ -224,8 +224,8 @@ def other_shapes_leg(torch, pypto_amd, dev):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=200)    # the device clocks settle over the first ~200 steps
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--counter-run", action="store_true",
                     help="for rocprofv3 --pmc: a few attention steps plus one device copy of COPY_MIB MiB "
@@ -316,7 +316,7 @@ def main():
         pypto_amd.sparse_attention_antiquant_d(sfa_d.query_nope, sfa_d.query_rope, packed, sel[i % ROT],
                                                sfa_d.block_table, sfa_d.kv_act_seqs, out_p, NQ, 1,
                                                sfa.softmax_scale, K, 128, sfa.max_blocknum_perbatch, None)
-    _, packed_avg_ms, _ = time_events(packed_step, max(args.steps // 2, 5), 5, torch)
+    _, packed_avg_ms, _ = time_events(packed_step, max(args.steps // 2, 5), 20, torch)
     sfa_step(0)
     packed_step(0)
     torch.cuda.synchronize()
@@ -330,7 +330,7 @@ def main():
         pypto_amd.lightning_indexer_decode(idx_queries[i % ROT], li_d.idx_query_scale, li_d.idx_key_cache,
                                            li_d.idx_key_scale, li_d.idx_weight, li_d.act_seq_key, li_d.block_table,
                                            res, None, None, K)
-    _, li2_avg_ms, _ = time_events(li_step, max(args.steps // 4, 5), 3, torch)
+    _, li2_avg_ms, _ = time_events(li_step, max(args.steps // 4, 5), 20, torch)
     li2_bytes = indexer_algorithmic_bytes(lengths, 4)
 
     li1 = gen_indexer_inputs(4, 1, config_lengths(1), selected_count=K, seed=1, variant="fp32").to(dev)
@@ -339,7 +339,7 @@ def main():
         pypto_amd.lightning_indexer_decode(li1.idx_query, li1.idx_query_scale, li1.idx_key_cache, li1.idx_key_scale,
                                            li1.idx_weight, li1.act_seq_key, li1.block_table, li1.topk_res, None, None,
                                            K)
-    _, li1_avg_ms, _ = time_events(li1_step, max(args.steps // 4, 5), 3, torch)
+    _, li1_avg_ms, _ = time_events(li1_step, max(args.steps // 4, 5), 20, torch)
     li1_bytes = indexer_algorithmic_bytes(config_lengths(1), 4)
 
     # ------------------------------------------------------------------ indexer prolog (projection stage)
