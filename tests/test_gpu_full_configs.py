@@ -181,3 +181,33 @@ def test_whole_decode_front_mla_prolog_indexer_prolog_indexer_attention(c_oracle
     assert torch.equal(q_int8.cpu(), torch.from_numpy(r_lip["q_int8"]))
     assert torch.equal(res.cpu(), want_idx), f"{int((res.cpu() != want_idx).sum())} index mismatches"
     check(out.cpu(), want_out, "whole decode front")
+
+
+# The shapes of the reference's own system-test cases for this operator
+# (framework/tests/st/operator/src/test_deepseek_v3.2_exp/gen_gather_selected_attention.py:358-450:
+# 128 heads, top-k 2048, blocks of 128; quantized and bf16 latent cache for each), on seeded synthetic data.
+@pytest.mark.parametrize("b,s1,act", [
+    (4, 2, [65536] * 4),
+    (4, 2, [666, 532, 768, 900]),
+    (32, 1, [511] * 32),
+    (1, 1, [2049]),
+    (1, 3, [2047]),
+    (128, 1, [8096] * 128),
+    (8, 1, [131072] * 8),
+    (4, 1, [666, 532, 768, 900]),
+    (8, 1, [666, 532, 768, 900, 5698, 2358, 324, 2048]),
+])
+def test_reference_system_test_shapes(c_oracle, b, s1, act):
+    from oracle import sfa_oracle as so
+    inp = gen_sfa_inputs(b, s1, 128, act, topk=2048, seed=100 + b + s1)
+    out = run_sfa(inp)
+    check(out, golden(c_oracle, inp), f"reference case b={b} s1={s1} act={act[0]}..")
+    # the bf16-cache branch on exactly the values the int8 cache de-quantises to: the same bits
+    d = inp.to(torch.device(DEV))
+    kn_bf16 = so.dequant_kn(inp.key_nope_2d, inp.k_nope_scales).to(DEV)
+    out_b = torch.full([b, s1, 128, 512], float("nan"), dtype=torch.bfloat16, device=DEV)
+    pypto_amd.sparse_flash_attention_quant_d(d.query_nope, d.query_rope, kn_bf16, d.key_rope_2d, None, d.topk_indices,
+                                             d.block_table, d.kv_act_seqs, out_b, 128, 1, inp.softmax_scale, 2048,
+                                             inp.block_size, inp.max_blocknum_perbatch, None)
+    torch.cuda.synchronize()
+    assert torch.equal(out_b.cpu().view(torch.int16), out.view(torch.int16))

@@ -45,6 +45,10 @@ def assert_exact(got, ref, what):
     (2, 1, [100, 1], 2048),            # fewer candidates than k: padded with -1
     (1, 4, [9000], 2048),              # s1 = 4
     (1, 1, [33], 16),                  # partial 32-key block
+    # the two shapes of the reference's own system tests
+    # (framework/tests/st/operator/src/test_deepseek_v3.2_exp/gen_lightning_indexer.py:374-376, 428-430)
+    (4, 1, [768, 4097, 8192, 131071], 2048),
+    (4, 2, [65536] * 4, 2048),
 ])
 def test_indexer_bit_exact(c_oracle, variant, b, s1, act, k):
     inp = gen_indexer_inputs(b, s1, act, selected_count=k, seed=7 * b + s1 + k, variant=variant)
