@@ -36,31 +36,12 @@ constexpr int PITCH = D + 8;      // LDS row pitch in bf16 elements (1168 B: row
 constexpr int KSTEPS = D / 16;    // 36 contraction steps of 16
 constexpr int DVB = DN / 32;      // 16 output blocks of 32 value channels
 
-// 8 int8 (two dwords of a 16-byte load) times one scale -> 8 bf16 as one 16-byte LDS store.
+// Four int8 (one dword) times one scale -> four bf16 in two registers.
 // x*sc is formed as fma(float(x + 128), sc, -128*sc): the byte is biased to unsigned so that a single
 // v_cvt_f32_ubyteN converts it, and the fused multiply-add rounds the exact product (x*sc) once, which
 // is bit-identical to the rounded multiply (128*sc is exact).
-__device__ __forceinline__ void dequant8(const int r0, const int r1, const float sc, uint16_t *dst)
+__device__ __forceinline__ u32x2 dequant4(const uint32_t r, const float sc, const float bias /* -128 * sc */)
 {
-    const float bias = -128.0f * sc;
-    u32x4 out;
-#pragma unroll
-    for (int w = 0; w < 2; ++w) {
-        const uint32_t v = (uint32_t)(w == 0 ? r0 : r1) ^ 0x80808080u;
-        const float f0 = __builtin_fmaf((float)(v & 0xffu), sc, bias);
-        const float f1 = __builtin_fmaf((float)((v >> 8) & 0xffu), sc, bias);
-        const float f2 = __builtin_fmaf((float)((v >> 16) & 0xffu), sc, bias);
-        const float f3 = __builtin_fmaf((float)(v >> 24), sc, bias);
-        out[2 * w] = pack_bf16x2(f0, f1);
-        out[2 * w + 1] = pack_bf16x2(f2, f3);
-    }
-    *reinterpret_cast<u32x4 *>(dst) = out;
-}
-
-// four bytes -> four bf16 in two registers
-__device__ __forceinline__ u32x2 dequant4(const uint32_t r, const float sc)
-{
-    const float bias = -128.0f * sc;
     const uint32_t v = r ^ 0x80808080u;
     const float f0 = __builtin_fmaf((float)(v & 0xffu), sc, bias);
     const float f1 = __builtin_fmaf((float)((v >> 8) & 0xffu), sc, bias);
@@ -393,6 +374,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // instructions (about three per product) hold the matrix pipeline up.
     constexpr int PER = (KPW + 7) / 8;             // keys of this wave per piece
     u32x2 praw[2][QUANT ? PER : 1], plow[QUANT ? PER : 1];
+    float pbias[QUANT ? PER : 1];
     float psc[2][QUANT ? PER : 1];
     auto fetch_piece = [&](const int piece, const int slot) {
 #pragma unroll
@@ -411,7 +393,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         for (int q = 0; q < PER; ++q) {
             const int i = piece * PER + q;
             if (i < KPW) {
-                const u32x2 c = dequant4(praw[piece & 1][q][hf], psc[piece & 1][q]);
+                if (hf == 0) pbias[q] = -128.0f * psc[piece & 1][q];
+                const u32x2 c = dequant4(praw[piece & 1][q][hf], psc[piece & 1][q], pbias[q]);
                 if (hf == 0) {
                     plow[q] = c;
                 } else {
@@ -487,7 +470,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                 }
 #pragma unroll
                 for (int i = 0; i < BATCH; ++i) {
-                    const u32x2 lo = dequant4(r[i][0], sc[i]), hi = dequant4(r[i][1], sc[i]);
+                    const float bias = -128.0f * sc[i];
+                    const u32x2 lo = dequant4(r[i][0], sc[i], bias), hi = dequant4(r[i][1], sc[i], bias);
                     const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
                     *reinterpret_cast<u32x4 *>(pool_b + emit_off + (tile * KT * PITCH * 2 + (i0 + i) * PITCH * 2)) = v;
                 }
@@ -522,6 +506,21 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // inside the loop the only outstanding vector-memory operations are the gathers of later tiles and
     // the compiler's wait counts do not serialise them with the matrix products.
     if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);    // vmcnt(0), expcnt and lgkmcnt unconstrained
+
+    // Scores are scaled inside the exponent (one multiply-add per key).  That wants a positive scale: the
+    // sign of a negative one moves into Q^T (exact), and a zero one becomes the smallest normal number,
+    // under which every finite score still scales to an exponent that rounds to the same probabilities.
+    float sc_log2 = p.scale_log2;
+    if (sc_log2 < 0.f) {
+        sc_log2 = -sc_log2;
+#pragma unroll
+        for (int i = 0; i < KSTEPS; ++i) {
+            u32x4 v = __builtin_bit_cast(u32x4, qf[i]);
+            v ^= 0x80008000u;
+            qf[i] = __builtin_bit_cast(bf16x8, v);
+        }
+    }
+    if (sc_log2 == 0.f) sc_log2 = 1.17549435e-38f;
 
     // One tile.  For the int8 cache the parity of the tile number is a compile-time constant (the loop
     // below runs two tiles per trip), so every LDS address in here is a per-lane base plus an immediate
@@ -573,15 +572,14 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             for (int r = 0; r < 16; ++r)
                 if (kt + 8 * (r >> 2) + 4 * half + (r & 3) >= k_end) s[r] = -INFINITY;
         }
+        // the scale is positive here (its sign went into Q^T), so the largest raw score gives the largest
+        // scaled one and the scaling itself is folded into the exponent's multiply-add
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            s[r] *= p.scale_log2;
-            mx = fmaxf(mx, s[r]);
-        }
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
         {
             float lo, hi;
             both_halves(mx, lo, hi);
-            mx = fmaxf(lo, hi);
+            mx = fmaxf(lo, hi) * sc_log2;
         }
         // The reference max follows the true max lazily: probabilities may reach 2^RESCALE_TAU, which
         // fp32 sums and bf16 P hold without loss, and the accumulators are rescaled only on a jump.
@@ -594,7 +592,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         float lsum = 0.f;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            s[r] = __builtin_amdgcn_exp2f(s[r] - m_new);      // v_exp_f32; exp2(-inf) = 0
+            s[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc_log2, -m_new));      // v_exp_f32; exp2(-inf) = 0
             lsum += s[r];
         }
         m_run = m_new;
@@ -614,7 +612,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         auto softmax_tail = [&](const int part) {
 #pragma unroll
             for (int r = 8 + 4 * part; r < 12 + 4 * part; ++r) {
-                s[r] = __builtin_amdgcn_exp2f(s[r] - m_new);
+                s[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc_log2, -m_new));
                 lsum += s[r];
             }
             if (part == 1) {

@@ -204,3 +204,14 @@ def test_bf16_latent_cache_branch(n_q, b, s1, act, topk):
                              inp.actual_seq, inp.block_size, inp.softmax_scale, inp.topk, is_kn_quant=False)
     check(out, ref, f"bf16 cache nq={n_q} b={b} s1={s1}")
     assert torch.equal(out.view(torch.int16), run_op(inp).view(torch.int16))
+
+
+@pytest.mark.parametrize("scale", [-0.0416666679084301, 0.0, 0.25])
+def test_softmax_scale_of_any_sign(scale):
+    """The kernel scales scores inside the exponent and wants a positive factor: a negative one moves its
+    sign into the query, a zero one gives uniform weights.  All three against the golden, with key splits."""
+    inp = gen_sfa_inputs(2, 1, 128, [3000, 200], topk=512, seed=41)
+    inp.softmax_scale = scale
+    ref = oracle(inp)
+    check(run_op(inp), ref, f"scale={scale}")
+    check(run_op(inp, num_splits=4), ref, f"scale={scale}, 4 splits")
