@@ -343,8 +343,15 @@ def main():
     li1_bytes = indexer_algorithmic_bytes(config_lengths(1), 4)
 
     # ------------------------------------------------------------------ indexer prolog (projection stage)
-    prolog = prolog_leg(torch, dev, pypto_amd)
-    mla_prolog = mla_prolog_leg(torch, dev, pypto_amd)
+    # the side legs must not cost the headline line: a failure there is reported in its field
+    def side_leg(fn):
+        try:
+            return fn(torch, dev, pypto_amd)
+        except Exception as e:                                # noqa: BLE001 -- reported, not swallowed
+            torch.cuda.synchronize()
+            return {"error": f"{type(e).__name__}: {e}"}
+    prolog = side_leg(prolog_leg)
+    mla_prolog = side_leg(mla_prolog_leg)
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
