@@ -432,7 +432,13 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     int srow[REQ_PER_GROUP];
     auto group_pre = [&](const int u, const int slot, const int kt2, const int slot2) {
         if (!QUANT) return;
-        if (u % 2 == 0 && u / 2 < 8) fetch_piece(u / 2, slot);
+        if (u == 1) {
+            // the next tile's requests went out during the previous tile's products; the wait for the last
+            // of them comes after this tile's first products have been issued
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            asm volatile("" ::: "memory");
+        }
+        if (u % 2 == 1 && u / 2 < 8) fetch_piece(u / 2, slot);
         if (u == 15) fetch_rope(slot);
 #pragma unroll
         for (int j = 0; j < REQ_PER_GROUP; ++j) {
@@ -447,8 +453,11 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     };
     auto group_post = [&](const int u, const int tile) {
         if (QUANT) {
-            if (u >= 1) emit_half(tile, (u - 1) / 2, (u - 1) % 2);
-            if (u == 16) emit_rope(tile);
+            if (u >= 2) emit_half(tile, (u - 2) / 2, (u - 2) % 2);
+            if (u == 16) {
+                emit_half(tile, 7, 1);
+                emit_rope(tile);
+            }
         } else if (u == KSTEPS / 4) {
             emit_rope(tile);
         }
@@ -531,13 +540,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
         // next tile (or a padding tile) of the bf16 cache, the tile after it of the int8 cache: in flight
         // during the products
-        if (QUANT) {
-            // the next tile's requests went out during the previous tile's products: staged by now
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            asm volatile("" ::: "memory");
-        } else {
-            issue_loads(kt + KT, nxt_tile);
-        }
+        if (!QUANT) issue_loads(kt + KT, nxt_tile);
 
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
