@@ -187,6 +187,57 @@ def mla_prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=10, replays=10):
             "hbm_frac": byt / (us * 1e-6) / 1e9 / PEAK_HBM_GBS}
 
 
+def fused_prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=10, replays=10):
+    """One pass of mla_indexer_prolog_quant_d (MLA prolog, then the indexer prolog on its query latent), timed
+    like the two legs above: a HIP graph of `calls` passes, each with its own copy of all seven weight tensors."""
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
+    m = gen_mla_prolog_inputs(b, s1, [4096] * b, seed=0).to(dev)
+    ip = gen_indexer_prolog_inputs(b, s1, [4096] * b, seed=0).to(dev)
+    t, n, ql = b * s1, m.w_uk.shape[0], m.w_dq.shape[1]
+    ni = ip.w_proj.shape[1]
+    outs_m = (torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev), torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev),
+              m.kv_cache, m.kr_cache, m.k_scale_cache)
+    outs_i = (torch.empty([t, ni, 128], dtype=torch.int8, device=dev), torch.empty([t, ni, 1], dtype=torch.float16, device=dev),
+              ip.k_cache, ip.k_cache_scale, torch.empty([t, ni], dtype=torch.float16, device=dev))
+    sets = [(m.w_dq.clone(), m.w_uq_qr.clone(), m.w_uk.clone(), m.w_dkv_kr.clone(), ip.w_qb.clone(), ip.wk.clone(),
+             ip.w_proj.clone()) for _ in range(calls)]
+
+    def one(i=0):
+        wdq, wuq, wuk, wdkv, wqb, wk, wproj = sets[i]
+        pypto_amd.mla_indexer_prolog_quant_d(
+            m.token_x, wdq, wuq, m.dequant_scale, wuk, wdkv, m.gamma_cq, m.gamma_ckv, m.cos, m.sin, m.cache_index,
+            m.kv_cache, m.kr_cache, m.k_scale_cache, wqb, ip.w_qb_scale, wk, wproj, ip.ln_gamma_k, ip.ln_beta_k,
+            ip.hadamard_q, ip.hadamard_k, ip.k_cache, ip.k_cache_scale, *outs_m, *outs_i, 1e-5, 1e-5, "PA_BSND", None,
+            None, None, None)
+    for _ in range(3):
+        one()
+    torch.cuda.synchronize()
+    mode = "hip graph replay"
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(calls):
+                one(i)
+        run = g.replay
+    except Exception:                      # noqa: BLE001 -- capture support varies; eager timing still valid
+        mode = "eager calls (host time included)"
+
+        def run():
+            for i in range(calls):
+                one(i)
+    run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (calls * replays)
+    return {"workload": f"b={b} s={s1} (t={t}) MLA prolog ({n} heads) + indexer prolog ({ni} heads)", "us_per_pass": us,
+            "timing": mode + f", {calls} weight sets in rotation"}
+
+
 def other_shapes_leg(torch, pypto_amd, dev):
     """configs[3] and configs[4] through the same operators (parity of both is a GPU test): step time and the
     fraction of the dense bf16 peak their algorithmic flops reach.  Row (b, s) attends
@@ -352,6 +403,7 @@ def main():
             return {"error": f"{type(e).__name__}: {e}"}
     prolog = side_leg(prolog_leg)
     mla_prolog = side_leg(mla_prolog_leg)
+    fused_prolog = side_leg(fused_prolog_leg)
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
@@ -403,6 +455,7 @@ def main():
                     "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes, "scale_dtype": "fp32", "weight_dtype": "bf16"},
         "indexer_prolog": prolog,
         "mla_prolog": mla_prolog,
+        "mla_indexer_prolog": fused_prolog,
         "cpu_baseline": cpu,
     }
     if args.other_shapes:
