@@ -88,7 +88,14 @@ extern "C" {
  * (the reference reads unchecked); their contribution is unspecified.
  *
  * Constraints: n_kv == 1, topk >= 1, block_size >= 1, nq >= 1.
- * num_splits: how many workgroups share one query row's keys (0 = choose).
+ * Alignment: query, cache, output and workspace pointers 16 bytes (a contiguous
+ * torch view with a storage offset may not be), the int32 tensors 4 bytes.
+ * num_splits: how many workgroups share one query row's keys (0 = choose from
+ * the device's compute-unit count).  When a row is split, each split's result
+ * travels as fp16 normalised by the split's own row sum: de-quantised cache
+ * values must stay below 65504 in magnitude (always true of int8 * scale for
+ * sane scales; for the bf16 cache of pto_sfa_bf16kv_launch larger values give
+ * inf/NaN unless num_splits == 1).
  */
 typedef struct PtoSfaQuantArgs {
     const void *query_nope;
@@ -184,7 +191,9 @@ int pto_sa_antiquant_launch(const PtoSaAntiquantArgs *args, void *hip_stream);
  * ascending), padded with -1.
  *
  * Constraints: n_heads == 64, head_dim == 128, 1 <= selected_count <= 2048,
- * max_blocknum_perbatch * block_size <= 131072, block_size a multiple of 32.
+ * max_blocknum_perbatch * block_size <= 131072, block_size a multiple of 32,
+ * t <= 65535.  Alignment: idx_query, idx_key_cache and workspace 16 bytes, the
+ * int32 tensors 4 bytes, scales and weights their element size.
  */
 typedef struct PtoLiDecodeArgs {
     const int8_t *idx_query;

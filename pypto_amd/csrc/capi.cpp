@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -27,19 +28,29 @@ int fail(int code, const char *fmt, ...)
     return code;
 }
 
+}  // namespace
+
+namespace pto {
+// compute units of the current device (one query per device ordinal, then cached)
 int cu_count()
 {
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cached = n;
-        else
-            cached = 256;
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<int> cached[MAX_DEVICES];
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (dev >= 0 && dev < MAX_DEVICES) {
+        n = cached[dev].load(std::memory_order_relaxed);
+        if (n > 0) return n;
     }
-    return cached;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    if (dev >= 0 && dev < MAX_DEVICES) cached[dev].store(n, std::memory_order_relaxed);
+    return n;
 }
+}  // namespace pto
+
+namespace {
+
+using pto::cu_count;
 
 struct SfaPlan {
     int waves;
@@ -58,7 +69,8 @@ int sfa_check(const PtoSfaQuantArgs *a)
     if (a->block_size < 1 || a->max_blocknum_perbatch < 1)
         return fail(PTO_E_INVALID_ARG, "sfa: block_size and max_blocknum_perbatch must be >= 1");
     if (a->kv_rows < 1) return fail(PTO_E_INVALID_ARG, "sfa: kv_rows must be >= 1");
-    if (a->b * a->s1 > (1ll << 24) || a->nq > 65536 || a->topk > (1ll << 24) || a->kv_rows > 0x7fffffffll)
+    if (a->b > (1ll << 24) || a->s1 > (1ll << 24) || a->b * a->s1 > (1ll << 24) || a->nq > 65536 || a->topk > (1ll << 24) ||
+        a->kv_rows > 0x7fffffffll || a->block_size > (1ll << 30) || a->max_blocknum_perbatch > (1ll << 30))
         return fail(PTO_E_INVALID_ARG, "sfa: shape out of the supported range");
     if (a->num_splits < 0) return fail(PTO_E_INVALID_ARG, "sfa: num_splits must be >= 0");
     if (!std::isfinite(a->softmax_scale)) return fail(PTO_E_INVALID_ARG, "sfa: softmax_scale is not finite");
@@ -77,8 +89,10 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
     int ns = a->num_splits;
     if (ns == 0) {
         // fill the chip once; a split shorter than four tiles is all prologue
+        // (a size query on a host without a device plans for the 256 CUs of an MI355X; a launch there fails)
         const long long wgs = rows * pl.hgroups;
-        ns = (int)((cu_count() + wgs - 1) / wgs);
+        const int cus = cu_count() > 0 ? cu_count() : 256;
+        ns = (int)((cus + wgs - 1) / wgs);
         const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
         ns = ns > max_split ? max_split : ns;
     }
@@ -130,7 +144,20 @@ PtoSfaQuantArgs unpacked_view(const PtoSaAntiquantArgs *a)
 int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const uint8_t *kr, int kr_pitch, const uint8_t *ksc,
                 int ksc_pitch, void *hip_stream, bool kn_bf16 = false)
 {
+    if (cu_count() <= 0) return fail(PTO_E_NO_DEVICE, "sfa: no usable device is current");
     const SfaPlan pl = sfa_plan(a);
+    if (((long long)(a->b * a->s1) + 7) / 8 * 8 * pl.hgroups * pl.nsplit > 0x7fffffffll)
+        return fail(PTO_E_INVALID_ARG, "sfa: rows x head groups x key splits exceeds the largest launch");
+    {
+        const void *al16[] = {a->query_nope, a->query_rope, kn, kr, ksc, a->attention_out, a->workspace};
+        for (const void *ptr : al16)
+            if (reinterpret_cast<uintptr_t>(ptr) & 15)
+                return fail(PTO_E_INVALID_ARG, "sfa: query, cache, output and workspace pointers must be 16-byte aligned");
+        const void *al4[] = {a->topk_indices, a->block_table, a->kv_act_seqs};
+        for (const void *ptr : al4)
+            if (reinterpret_cast<uintptr_t>(ptr) & 3)
+                return fail(PTO_E_INVALID_ARG, "sfa: index, block-table and length pointers must be 4-byte aligned");
+    }
     const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
     if (need > 0 && (!a->workspace || a->workspace_bytes < need))
         return fail(PTO_E_WORKSPACE, "sfa: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
@@ -163,9 +190,13 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
     p.waves = pl.waves;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
     hipError_t e = pto::sfa_launch(p, static_cast<hipStream_t>(hip_stream));
+    if (e == hipErrorNoBinaryForGpu || e == hipErrorInvalidDeviceFunction)
+        return fail(PTO_E_NO_DEVICE, "sfa: the library holds gfx950 code only: %s", hipGetErrorString(e));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "sfa: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
 }
+
+constexpr long long LI_MAX_SEQ_HOST = pto::LI_MAX_SEQ;
 
 int li_check(const PtoLiDecodeArgs *a)
 {
@@ -180,7 +211,10 @@ int li_check(const PtoLiDecodeArgs *a)
     if (a->block_num < 1 || a->max_blocknum_perbatch < 1) return fail(PTO_E_INVALID_ARG, "li: block_num and max_blocknum_perbatch must be >= 1");
     if (a->max_blocknum_perbatch * a->block_size > pto::LI_MAX_SEQ)
         return fail(PTO_E_INVALID_ARG, "li: max_blocknum_perbatch * block_size exceeds %d", pto::LI_MAX_SEQ);
-    if (a->t > (1ll << 20) || a->block_num * a->block_size > 0x7fffffffll) return fail(PTO_E_INVALID_ARG, "li: shape out of the supported range");
+    if (a->t > (1ll << 20) || a->block_num > 0x7fffffffll || a->block_size > LI_MAX_SEQ_HOST || a->block_num * a->block_size > 0x7fffffffll)
+        return fail(PTO_E_INVALID_ARG, "li: shape out of the supported range");
+    if (a->t > pto::LI_MAX_BALANCED_TOKENS && a->t > 65535)
+        return fail(PTO_E_INVALID_ARG, "li: at most 65535 query tokens per launch (got %lld)", (long long)a->t);
     if (a->arith_variant != 0 && a->arith_variant != 1) return fail(PTO_E_INVALID_ARG, "li: arith_variant must be 0 or 1");
     if (a->arith_variant == 1 &&
         (a->q_scale_dtype != PTO_DT_FP16 || a->k_scale_dtype != PTO_DT_FP16 || a->weight_dtype != PTO_DT_FP16))
@@ -337,6 +371,22 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     const size_t need = li_ws_bytes(a);
     if (!a->workspace || a->workspace_bytes < need)
         return fail(PTO_E_WORKSPACE, "li: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+    if (cu_count() <= 0) return fail(PTO_E_NO_DEVICE, "li: no usable device is current");
+    {
+        const void *al16[] = {a->idx_query, a->idx_key_cache, a->workspace};
+        for (const void *ptr : al16)
+            if (reinterpret_cast<uintptr_t>(ptr) & 15)
+                return fail(PTO_E_INVALID_ARG, "li: query, key-cache and workspace pointers must be 16-byte aligned");
+        const void *al4[] = {a->act_seq_key, a->block_table, a->topk_res};
+        for (const void *ptr : al4)
+            if (reinterpret_cast<uintptr_t>(ptr) & 3)
+                return fail(PTO_E_INVALID_ARG, "li: length, block-table and result pointers must be 4-byte aligned");
+        const void *sc[] = {a->idx_query_scale, a->idx_key_scale, a->idx_weight};
+        const int sdt[] = {a->q_scale_dtype, a->k_scale_dtype, a->weight_dtype};
+        for (int i = 0; i < 3; ++i)
+            if (reinterpret_cast<uintptr_t>(sc[i]) & (sdt[i] == PTO_DT_FP32 ? 3 : 1))
+                return fail(PTO_E_INVALID_ARG, "li: scale and weight pointers must be aligned to their element size");
+    }
 
     pto::LiParams p;
     p.q = a->idx_query;

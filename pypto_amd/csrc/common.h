@@ -72,6 +72,10 @@ __device__ __forceinline__ void dma4(const void *gaddr, const uint32_t lds_dst)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
 }
 // s_waitcnt immediate for "at most n vector-memory operations outstanding" (the other counters unconstrained)
+// compute units of the current device, cached per device ordinal; 0 if the device cannot be asked
+// (host side, defined with the C ABI)
+int cu_count();
+
 constexpr int vmcnt_imm(const int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
 }  // namespace pto

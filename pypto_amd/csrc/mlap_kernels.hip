@@ -372,18 +372,6 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
             p.q_nope[((size_t)(t0 + t) * p.n_heads + head) * MLAP_KV + colbase + l] = (uint16_t)(pack_bf16x2(acc[t], 0.f) & 0xffffu);
 }
 
-int cu_count()
-{
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cached = n;
-        else
-            cached = 256;
-    }
-    return cached;
-}
 
 }  // namespace
 
@@ -404,7 +392,9 @@ hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
     // as many workgroups as fit at once (by their LDS), every one with the same number of jobs where possible
     const int steps = p.q_lora / QPROJ_KSPLIT / 32;
     const int lds = steps == 12 ? qproj_lds_bytes<6>() : (steps == 8 ? qproj_lds_bytes<4>() : qproj_lds_bytes<2>());
-    const int slots = cu_count() * (160 * 1024 / lds);
+    const int cus = cu_count();
+    if (cus <= 0) return hipErrorNoDevice;
+    const int slots = cus * (160 * 1024 / lds);
     const int rounds = (qjobs + slots - 1) / slots;
     const dim3 qgrid((unsigned)((qjobs + rounds - 1) / rounds));
     switch (steps) {

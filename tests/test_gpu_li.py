@@ -107,6 +107,21 @@ def test_long_runs_wide_block_table(c_oracle):
     assert_exact(run_op(inp), oracle(inp, c_oracle), "wide block table")
 
 
+@pytest.mark.parametrize("b,s1", [
+    (100, 1),     # balanced run mapping, rows 1.. of the token table (tokens 64 and up)
+    (40, 4),      # the same with four query tokens per sequence
+    (130, 4),     # 520 tokens: past the balanced mapping, one grid row per token
+])
+def test_many_query_tokens_short_sequences(c_oracle, b, s1):
+    """More query tokens than one row of the score kernel's token table holds, and more than the balanced
+    mapping takes at all; short ragged sequences so the oracle stays cheap."""
+    g = torch.Generator().manual_seed(1000 + b)
+    act = [int(x) for x in torch.randint(s1, 700, [b], generator=g)]
+    act[0], act[-1] = 699, s1                      # a long first and the shortest possible last sequence
+    inp = gen_indexer_inputs(b, s1, act, selected_count=128, seed=b + s1, variant="fp16")
+    assert_exact(run_op(inp), oracle(inp, c_oracle), f"b={b} s1={s1}")
+
+
 def test_small_pages_and_small_k(c_oracle):
     """32-key pages (every block of a pair on its own page) and small selection counts."""
     for k, act in ((1, [5000, 70]), (17, [2500, 31]), (512, [700, 513])):
