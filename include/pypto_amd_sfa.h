@@ -125,6 +125,24 @@ int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *args, size_t *bytes);
 int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
 
 /*
+ * pto_sfa_quant_launch for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc): it has no
+ * counterpart in the reference.  The partial results of the key splits go to an
+ * array built into the library (PTO_SFA_STATIC_SCRATCH_BYTES per GPU, held until
+ * the process ends) instead of a workspace; args->workspace and workspace_bytes
+ * are ignored.  Nothing is allocated or freed; the first call on a device looks
+ * the array's device address up.  A shape whose splits need more than the array
+ * holds is refused with PTO_E_WORKSPACE (every BASELINE decode shape fits: 32
+ * rows x 8 splits and 128 rows x 2 splits of 128 heads take 33.8 MB).
+ * All calls on one GPU share the array: calls whose execution may overlap (two
+ * streams, two threads) race on it and must use pto_sfa_quant_launch with
+ * workspaces of their own instead.  Nothing in the array has to be cleared
+ * between calls: every split writes its partial before it is read.
+ */
+#define PTO_SFA_STATIC_SCRATCH_BYTES ((size_t)40 << 20)
+int pto_sfa_quant_launch_static(const PtoSfaQuantArgs *args, void *hip_stream);
+
+/*
  * The non-quantized branch of the same operator (key_nope_2d not int8,
  * sparse_flash_attention_quant_impl.py:149-153 and 199-202 in the reference
  * example): key_nope_2d is [kv_rows, 512] bf16 and is used as it is,

@@ -9,11 +9,19 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "li_kernels.h"
 #include "lip_kernels.h"
 #include "mlap_kernels.h"
 #include "sfa_kernels.h"
+
+// Scratch memory of pto_sfa_quant_launch_static: the partial results of the key splits live here
+// instead of in a caller workspace.  One copy per GPU the library's code object is loaded on, held
+// until the process ends.  In host code the name below is only a handle; the device address is asked
+// for once per device (scratch_of) and that pointer is what the kernels get.
+constexpr size_t SFA_STATIC_SCRATCH_BYTES = (size_t)40 << 20;
+static __device__ __align__(256) unsigned char scratch[SFA_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -51,6 +59,32 @@ int cu_count()
 namespace {
 
 using pto::cu_count;
+
+// device address of this device's copy of the scratch array (NULL and *err set on failure)
+void *scratch_of(int dev, hipError_t *err)
+{
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<void *> ptrs[MAX_DEVICES];
+    static std::mutex mu;
+    *err = hipSuccess;
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    void *p = ptrs[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    std::lock_guard<std::mutex> lock(mu);
+    p = ptrs[dev].load(std::memory_order_relaxed);
+    if (p) return p;
+    void *addr = nullptr;
+    *err = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));     // the current device is dev (checked by the caller)
+    if (*err != hipSuccess || !addr) {
+        if (*err == hipSuccess) *err = hipErrorInvalidSymbol;
+        return nullptr;
+    }
+    ptrs[dev].store(addr, std::memory_order_release);
+    return addr;
+}
 
 struct SfaPlan {
     int waves;
@@ -317,6 +351,32 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *a, void *hip_stream)
         !a->block_table || !a->kv_act_seqs || !a->attention_out)
         return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
     return sfa_enqueue(a, static_cast<const int8_t *>(a->key_nope_2d), 512, static_cast<const uint8_t *>(a->key_rope_2d), 128,
+                       static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream);
+}
+
+int pto_sfa_quant_launch_static(const PtoSfaQuantArgs *a, void *hip_stream)
+{
+    int rc = sfa_check(a);
+    if (rc != PTO_OK) return rc;
+    if (!a->query_nope || !a->query_rope || !a->key_nope_2d || !a->key_rope_2d || !a->k_nope_scales || !a->topk_indices ||
+        !a->block_table || !a->kv_act_seqs || !a->attention_out)
+        return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
+    const SfaPlan pl = sfa_plan(a);
+    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
+    if (need > SFA_STATIC_SCRATCH_BYTES)
+        return fail(PTO_E_WORKSPACE,
+                    "sfa: the key splits of this shape need %zu bytes of scratch, the built-in array holds %zu; use "
+                    "pto_sfa_quant_launch with a workspace, or fewer splits",
+                    need, SFA_STATIC_SCRATCH_BYTES);
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(PTO_E_NO_DEVICE, "sfa: no current device: %s", hipGetErrorString(e));
+    void *ptr = scratch_of(dev, &e);
+    if (!ptr) return fail(PTO_E_NO_DEVICE, "sfa: the scratch array has no address on device %d: %s", dev, hipGetErrorString(e));
+    PtoSfaQuantArgs q = *a;
+    q.workspace = ptr;
+    q.workspace_bytes = SFA_STATIC_SCRATCH_BYTES;
+    return sfa_enqueue(&q, static_cast<const int8_t *>(a->key_nope_2d), 512, static_cast<const uint8_t *>(a->key_rope_2d), 128,
                        static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream);
 }
 
