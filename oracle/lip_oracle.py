@@ -119,7 +119,11 @@ def pair_tree_sum(v: np.ndarray) -> np.ndarray:
 
 def q_linear(q_norm: np.ndarray, w_qb: np.ndarray) -> np.ndarray:
     """Exact int8 x int8 matmul, [T,K] x [K,N] -> int32 (|sum| <= K * 2**14 < 2**31)."""
-    return (q_norm.astype(np.int64) @ w_qb.astype(np.int64)).astype(np.int32)
+    # through the float64 matrix product: every product is below 2**14 and every partial sum below 2**31, all
+    # exactly representable, so the sum is exact whatever order the library takes (an integer matmul in
+    # numpy is the same numbers, two orders of magnitude slower)
+    acc = q_norm.astype(np.float64) @ w_qb.astype(np.float64)
+    return acc.astype(np.int64).astype(np.int32)
 
 
 def rope_first(x: np.ndarray, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:

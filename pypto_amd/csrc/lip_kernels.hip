@@ -360,7 +360,7 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipPar
         const float mean = __fmul_rn(pair_tree_sum(v0, v1), 1.0f / LIP_DIM);
         const float d0 = __fsub_rn(v0, mean), d1 = __fsub_rn(v1, mean);
         const float var = __fmul_rn(pair_tree_sum(__fmul_rn(d0, d0), __fmul_rn(d1, d1)), 1.0f / LIP_DIM);
-        const float sd = __fsqrt_rn(__fadd_rn(var, p.eps));
+        const float sd = __builtin_sqrtf(__fadd_rn(var, p.eps));   // correctly rounded (__fsqrt_rn is the 1-ulp hardware root here)
         v0 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d0, sd), __uint_as_float(gm << 16)), __uint_as_float(bt << 16)));
         v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(gm & 0xffff0000u)), __uint_as_float(bt & 0xffff0000u)));
         rope_pair(v0, v1, rc, rs, l);

@@ -192,7 +192,7 @@ __global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapPara
     if (w < nslab) {
         float s = 0.f;
         for (int j = 0; j < nslab; ++j) s = __fadd_rn(s, slabsum[j]);
-        const float d = __fsqrt_rn(__fadd_rn(s, kvtype ? p.eps_ckv : p.eps_cq));
+        const float d = __builtin_sqrtf(__fadd_rn(s, kvtype ? p.eps_ckv : p.eps_cq));   // correctly rounded (__fsqrt_rn is the 1-ulp hardware root here)
         const uint32_t gm = reinterpret_cast<const uint32_t *>(kvtype ? p.gamma_ckv : p.gamma_cq)[w * 64 + l];
         y0 = bf16_round_f32(__fmul_rn(__fdiv_rn(v0, d), __uint_as_float(gm << 16)));
         y1 = bf16_round_f32(__fmul_rn(__fdiv_rn(v1, d), __uint_as_float(gm & 0xffff0000u)));

@@ -99,3 +99,15 @@ def test_prolog_mtp_batch_t128():
     inp = gen_indexer_prolog_inputs(32, 4, [2048 + 17 * i for i in range(32)], seed=2)
     ref = lo.indexer_prolog_ref(*inp.input_tensors())
     assert_exact(run_op(inp), ref, "b32_s1_4")
+
+
+@pytest.mark.parametrize("b,s1,act,what", [
+    (128, 4, [8192] * 128, "b128_s1_4_s2_8k"),       # 512 tokens
+    (1, 4096, [65536], "b1_s1_4k_s2_64k"),           # 4096 tokens of one sequence (prefill)
+])
+def test_prolog_reference_large_cases(b, s1, act, what):
+    """The reference's "large" cases (deepseekv32_lightning_indexer_prolog_quant.py:470-509) at the model's
+    full projection sizes: the decode kernels walk the token blocks, so the bar stays bit-exact."""
+    inp = gen_indexer_prolog_inputs(b, s1, act, seed=b + s1)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert_exact(run_op(inp), ref, what)

@@ -78,6 +78,14 @@ def test_mla_prolog_reference_case_b4_s2():
     assert np.abs(got["k_scale_cache"].reshape(-1, 4)[rows] - ks.numpy()).max() <= 2.5e-5 + 0.005 * np.abs(ks.numpy()).max()
 
 
+def test_mla_prolog_prefill_t512():
+    """mla_prolog_quant_p on one sequence of 512 tokens at full size, the largest case the reference carries for
+    this operator (deepseekv32_mla_indexer_prolog_quant.py:1049-1050, t_512): bit-exact like the decode cases."""
+    inp = gen_mla_prolog_inputs(1, 512, [4096], seed=21)
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    assert_exact(run_op(inp, (1e-5, 1e-5), prefill=True), ref, "t_512 prefill")
+
+
 def test_mla_prolog_separate_cache_output_skipped_indices_and_repeatability():
     inp = gen_mla_prolog_inputs(2, 2, [300, 129], seed=5, h=256, q_lora_rank=512, n_heads=4)
     inp.cache_index[1] = -1
