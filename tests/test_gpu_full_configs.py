@@ -69,6 +69,34 @@ def test_config3_two_query_tokens_per_sequence(c_oracle):
     check(out, golden(c_oracle, inp), "cfg3")
 
 
+def test_config3_chain_indexer_then_attention(c_oracle):
+    """B=64, S1=2, KV 4096..32768, chained at full size: the indexer scores both query tokens of a sequence
+    (the first may not select the last position, the second may: eff_seq = act - (S1-1-s)), its indices must
+    equal the golden's bit for bit, and the attention over them (cur_seq = min(act - S1 + 1 + s, topk)) must
+    match the golden within tolerance."""
+    B, S1, K = 64, 2, 2048
+    lengths = config_lengths(3, seed=3)
+    li = gen_indexer_inputs(B, S1, lengths, selected_count=K, seed=12, variant="fp32")
+    sfa = gen_sfa_inputs(B, S1, 128, lengths, topk=K, seed=13, block_table=li.block_table, block_num=li.block_num,
+                         topk_indices=torch.zeros([B * S1, K], dtype=torch.int32))
+    d = li.to(torch.device(DEV))
+    pypto_amd.lightning_indexer_decode(d.idx_query, d.idx_query_scale, d.idx_key_cache, d.idx_key_scale, d.idx_weight,
+                                       d.act_seq_key, d.block_table, d.topk_res, None, None, K)
+    torch.cuda.synchronize()
+    want = c_oracle.li_decode(li.idx_query, li.idx_query_scale, li.idx_key_cache, li.idx_key_scale, li.idx_weight,
+                              li.act_seq_key, li.block_table, K)
+    got = d.topk_res.cpu()
+    assert torch.equal(got, want), f"{int((got != want).sum())} index mismatches"
+    # the causal rule, seen in the indices themselves: token 0 of a sequence never holds its last position,
+    # token 1 may (and every position is below the token's effective length)
+    g = got.reshape(B, S1, K)
+    for b, n in enumerate(lengths):
+        assert int(g[b, 0].max()) <= n - 2 and int(g[b, 1].max()) <= n - 1
+    sel = d.topk_res.reshape(B * S1, K).contiguous()
+    out = run_sfa(sfa, topk_indices=sel)
+    check(out, golden(c_oracle, sfa, topk_indices=sel.cpu()), "cfg3 chain")
+
+
 def test_config4_prefill_4096_tokens(c_oracle):
     """B=1, S1=4096, KV 4096: row s sees min(s + 1, 2048) keys.  Every row against the golden; the first
     row, which sees one key, must be that key's de-quantised value row exactly."""
