@@ -261,9 +261,9 @@ int li_check(const PtoLiDecodeArgs *a)
 
 size_t li_ws_bytes(const PtoLiDecodeArgs *a)
 {
-    // score rows [t, max_blocknum_perbatch*block_size] fp32
+    // score rows [t, max_blocknum_perbatch*block_size] fp32, then one sampled score per 16 positions
     const size_t stride = (size_t)a->max_blocknum_perbatch * a->block_size;
-    return (size_t)a->t * stride * sizeof(float);
+    return (size_t)a->t * (stride + stride / pto::LI_SAMPLE_GROUP) * sizeof(float);
 }
 
 int lip_check(const PtoLiPrologQuantArgs *a)
@@ -466,6 +466,7 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.k = (int)a->selected_count;
     p.score_stride = (long long)a->max_blocknum_perbatch * a->block_size;
     p.scores = static_cast<float *>(a->workspace);
+    p.sample = p.scores + (size_t)a->t * p.score_stride;
     p.q_dt = a->q_scale_dtype;
     p.k_dt = a->k_scale_dtype;
     p.w_dt = a->weight_dtype;

@@ -10,6 +10,7 @@ constexpr int LI_MAX_SEQ = 128 * 1024;  // longest key sequence
 constexpr int LI_HEADS = 64;
 constexpr int LI_DIM = 128;
 constexpr int LI_MAX_BALANCED_TOKENS = 512; // most query tokens the balanced run mapping of the score kernel handles
+constexpr int LI_SAMPLE_GROUP = 16;        // the score kernel leaves one sampled score per this many positions
 constexpr int LI_MAX_PAIRS_PER_WAVE = 32;  // a wave keeps one cache-row index per 32-key block of its run in a lane
 
 struct LiParams {
@@ -22,6 +23,7 @@ struct LiParams {
     const int32_t *bt;      // [B, maxblk]
     int32_t *topk_res;      // [T, k]
     float *scores;          // workspace [T, score_stride]
+    float *sample;          // workspace [T, score_stride / 16]: one score of every 16 consecutive positions
     long long score_stride;
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes

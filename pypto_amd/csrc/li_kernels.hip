@@ -166,6 +166,15 @@ __device__ __forceinline__ uint32_t dequant_relu_weight(const uint32_t x, const 
     return __builtin_bit_cast(uint32_t, v * __builtin_bit_cast(f16x2, w));
 }
 
+// Sample for the select: of every 16 consecutive positions that all lie inside the sequence, the score
+// of one (picked by a hash of the group number) is also written to a compact array, so that the select
+// kernel finds a sample of the row in a few contiguous cache lines instead of thousands of scattered ones.
+__device__ __forceinline__ bool sample_lane(const int pos, const int cur)
+{
+    const uint32_t g = (uint32_t)pos >> 4;
+    return (uint32_t)(pos & 15) == ((g * 2654435761u) >> 28) && (int)(16u * g + 15u) < cur;
+}
+
 constexpr int SC_PAIR_BYTES = 64 * LI_DIM;     // key rows of one staged pair of 32-key blocks
 constexpr int SC_BUF_BYTES = SC_PAIR_BYTES + 256;   // + the 64 key scales (one dword per lane)
 
@@ -339,6 +348,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
     }
 
     float *srow = p.scores + (size_t)t * p.score_stride;
+    float *smp = p.sample + (size_t)t * (p.score_stride / LI_SAMPLE_GROUP);
     // 2^-11 as a run-time value, so that it sits in a scalar register (the mix instructions take no literal)
     const float scale = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3a000000));
     // this lane's operand chunks of row j inside a staged block
@@ -424,6 +434,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             }
             const int pos = key0 + 64 * pr + l;
             if (pos < cur) srow[pos] = sum;
+            if (sample_lane(pos, cur)) smp[pos >> 4] = sum;
             return;
         }
 #pragma unroll
@@ -443,7 +454,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             }
         }
         const int pos = key0 + 64 * pr + l;
-        if (pos < cur) srow[pos] = __fmul_rn(sum, ksc);
+        const float sc = __fmul_rn(sum, ksc);
+        if (pos < cur) srow[pos] = sc;
+        if (sample_lane(pos, cur)) smp[pos >> 4] = sc;
     };
     for (int pr = 0; pr < npair; pr += 2) {
         trip(pr, 0);
@@ -658,7 +671,7 @@ __device__ void bitonic_sort_desc(unsigned long long *buf, const int width, cons
     __syncthreads();
 }
 
-constexpr int SEL_SAMPLE = 2048;   // most keys sampled from a row
+constexpr int SEL_SAMPLE = 4096;   // most keys sampled from a row
 constexpr int SEL_CAP = 8192;      // candidates (keys above the pivot) the fast path holds in LDS
 constexpr int SEL_STAGE = 4096;    // entries of the buckets down to the one holding the k-th best
 constexpr int SEL_RANK_MAX = 512;  // rows of at most k keys: ordered by counting up to this length, else sorted
@@ -697,7 +710,8 @@ constexpr int SEL_CHUNK = 32 * SEL_THREADS;   // scores one trip of the row scan
 
 // One workgroup per query token: a distribution-adaptive bucket select.  Every key is ordered by the
 // word (score image << 32) | ~position, a strict order, so ties need no special case.
-//   1. up to 2048 scores are sampled (one per stratum of the row, jittered).  A histogram of the
+//   1. up to 4096 scores are sampled: the score kernel left one score of every 16 positions (which of
+//      the 16, a hash of the group number decides) in a compact array.  A histogram of the
 //      sample over [sample min, sample max] gives the pivot: the lower edge of the bin in which the
 //      sample reaches rank r = r0 + 6*sqrt(r0) + 8, r0 = k*S/n.  With overwhelming probability at
 //      least k and at most SEL_CAP scores of the row lie at or above it;
@@ -762,17 +776,24 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_kernel(const LiParams p
 
     // ---- 1. sample: the loads go out first, then the first chunk of the row, so that one memory
     // latency covers both
-    const uint32_t S = n < SEL_SAMPLE ? (uint32_t)n : (uint32_t)SEL_SAMPLE;
-    float sx[2];
-    bool sval[2];
+    // (the score kernel left one score of every 16 positions in a compact array; a row longer than
+    // 16 * SEL_SAMPLE takes every other one).  Rows with hardly any full group go the general way.
+    const uint32_t s_full = (uint32_t)n / (uint32_t)LI_SAMPLE_GROUP;
+    if (s_full < 64u) {
+        select_streaming(p, t, hist, stage);                     // uniform: the whole workgroup goes
+        return;
+    }
+    const uint32_t sstep = s_full > (uint32_t)SEL_SAMPLE ? 2u : 1u;
+    const uint32_t S = s_full / sstep;
+    constexpr int SPT = SEL_SAMPLE / SEL_THREADS;
+    const float *smp = p.sample + (size_t)t * (p.score_stride / LI_SAMPLE_GROUP);
+    float sx[SPT];
+    bool sval[SPT];
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
+    for (int e = 0; e < SPT; ++e) {
         const uint32_t i = (uint32_t)(tid + e * SEL_THREADS);
         sval[e] = i < S;
-        // stratum i of the row is [i*n/S, (i+1)*n/S): products stay below 2^28
-        const uint32_t ic = sval[e] ? i : 0u;
-        const uint32_t lo = ic * (uint32_t)n / S, hi = (ic + 1u) * (uint32_t)n / S;
-        sx[e] = srow[lo + ((ic * 2654435761u) >> 16) % (hi - lo)];
+        sx[e] = smp[(sval[e] ? i : 0u) * sstep];
     }
     // the row as 16-byte vectors: thread tid holds vectors u*1024 + tid of a chunk.  The row buffer is
     // score_stride (a multiple of 32) long, so whole vectors stay inside it.
@@ -793,7 +814,7 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_kernel(const LiParams p
     {
         float mn = __builtin_inff(), mx = -__builtin_inff();
 #pragma unroll
-        for (int e = 0; e < 2; ++e)
+        for (int e = 0; e < SPT; ++e)
             if (sval[e]) { mn = fminf(mn, sx[e]); mx = fmaxf(mx, sx[e]); }
         mn = wave_min(mn);
         mx = wave_max(mx);
@@ -811,7 +832,7 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_kernel(const LiParams p
         const float range = smax - smin;
         const float sscale = range > 0.f ? (float)SEL_SBINS / range : 0.f;
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
+        for (int e = 0; e < SPT; ++e) {
             if (sval[e]) {
                 const uint32_t sb = (uint32_t)fmaxf((sx[e] - smin) * sscale, 0.f);
                 atomicAdd(&shist[sb < (uint32_t)SEL_SBINS ? sb : (uint32_t)SEL_SBINS - 1u], 1u);

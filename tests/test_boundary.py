@@ -51,7 +51,7 @@ def test_pybind_workspace_and_argument_errors():
     # 32 rows x 8 splits x 128 heads x (512 fp16 + 2 fp32)
     assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 20, 0.04, 8) == 32 * 8 * 128 * (512 * 2 + 8)
     assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 0      # no split needed
-    assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * 32768 * 4
+    assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * (32768 + 2048) * 4
     # prolog: 4 int32 partial projections [t, 8192] + 112 block sums [t, 192] fp32
     assert C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 64, 1 << 20) == 4 * 8 * 8192 * 4 + 112 * 8 * 192 * 4
     with pytest.raises(ValueError):
