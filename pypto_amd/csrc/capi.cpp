@@ -473,14 +473,24 @@ int pto_li_decode_launch(const PtoLiDecodeArgs *a, void *hip_stream)
     p.variant = a->arith_variant;
     {   // A wave pays three dependent memory latencies before its first pair, so runs are made as long
         // as still leaves every SIMD two rounds of two waves; at most 32 pairs (2048 keys) per wave.
-        const long long pairs = (long long)a->t * ((p.score_stride + 63) / 64);
+        // Two query tokens of a sequence share a key pass (half the key bytes, the same arithmetic) when
+        // there are two and the pass then still has several rounds of work for every resident wave; a
+        // small batch is bound by latency, not bytes, and keeps one token per wave for twice the waves.
+        int nt = 1;
+        if (p.S1 >= 2 && p.variant == 0) {
+            const long long pairs2 = (long long)p.B * ((p.S1 + 1) / 2) * ((p.score_stride + 63) / 64);
+            if (pairs2 >= 8ll * cu_count() * 8) nt = 2;
+        }
+        p.nt = nt;
+        const long long units = (long long)p.B * ((p.S1 + nt - 1) / nt);    // token groups that share a key pass
+        const long long pairs = units * ((p.score_stride + 63) / 64);
         long long ppw = pairs / ((long long)cu_count() * 4 * 4);
         p.ppw = (int)(ppw < 1 ? 1 : (ppw > pto::LI_MAX_PAIRS_PER_WAVE ? pto::LI_MAX_PAIRS_PER_WAVE : ppw));
-        // With few query tokens the kernel balances the runs itself from the actual lengths: one round
+        // With few units the kernel balances the runs itself from the actual lengths: one round
         // of resident waves (two workgroups per CU), more only if the longest possible input needs it.
-        p.balanced = a->t <= pto::LI_MAX_BALANCED_TOKENS;
+        p.balanced = units <= pto::LI_MAX_BALANCED_TOKENS;
         long long waves = (long long)cu_count() * 8;
-        const long long need = (pairs + pto::LI_MAX_PAIRS_PER_WAVE - 1) / pto::LI_MAX_PAIRS_PER_WAVE + 2 * a->t;
+        const long long need = (pairs + pto::LI_MAX_PAIRS_PER_WAVE - 1) / pto::LI_MAX_PAIRS_PER_WAVE + 2 * units;
         waves = waves > need ? waves : need;
         p.score_wgs = (int)((waves + 3) / 4);
     }

@@ -28,8 +28,9 @@ struct LiParams {
     int T, B, S1, bs, maxblk, nblocks, k;
     int q_dt, k_dt, w_dt;   // PTO_DT_* codes
     int ppw;                // 64-key block pairs per wave of the score kernel, <= LI_MAX_PAIRS_PER_WAVE
-    int balanced;           // score kernel sizes its runs from the sequence lengths (T <= LI_MAX_BALANCED_TOKENS)
+    int balanced;           // score kernel sizes its runs from the sequence lengths (units <= LI_MAX_BALANCED_TOKENS)
     int score_wgs;          // its launch size in workgroups of four waves when balanced
+    int nt;                 // query tokens of one sequence that a wave of the score kernel scores per key pass: 1 or 2
     int variant;            // 0: fp32 head factors applied after the ReLU; 1: fp16 scales applied before it (all tensors fp16)
 };
 

@@ -132,6 +132,18 @@ __device__ __forceinline__ float mul_f16_f32(const uint32_t packed, const float 
     return r;
 }
 
+// the same with the factor in a vector register (read from LDS)
+template <int HI>
+__device__ __forceinline__ float mul_f16_f32_v(const uint32_t packed, const float w)
+{
+    float r;
+    if (HI)
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(w));
+    else
+        asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(packed), "v"(w));
+    return r;
+}
+
 // x = fp16(relu(dot) / 2048) for two dots, packed.  v_fma_mixlo/mixhi_f16 scale in fp32 (exact: a power
 // of two) and round once to fp16; -|dot|/2048 rounds to a negative fp16 that the packed integer max
 // then clears, which equals clearing first.  scale = 2^-11 in a scalar register.
@@ -202,10 +214,17 @@ constexpr int SC_BUF_BYTES = SC_PAIR_BYTES + 256;   // + the 64 key scales (one 
 // framework/src/operator/models/deepseek_v3.2_exp/lightning_indexer.cpp:149-197): fp16(dot/2048) is
 // multiplied in fp16 by the head's query scale and by the key's scale before the ReLU, then in fp16 by
 // the head's weight; the fp32 head sum (h ascending) is the score.  All three tensors are fp16 then.
-template <int KDT, int VAR = 0>
+// NT = query tokens of one sequence a wave scores per key pass (1 or 2): the reference scores all s1 tokens of
+// a batch against a page in one matrix product (lightning_indexer_quant_impl.py:163-169, [S1*64, 128]); here
+// a "unit" is a pair of consecutive tokens of a sequence (the last unit of an odd s1 holds one), every staged
+// key row and scale serves both, and their per-head factors sit in LDS instead of scalar registers.
+template <int KDT, int VAR = 0, int NT = 1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void li_score_kernel(const LiParams p)
 {
     __shared__ __attribute__((aligned(16))) int8_t kstage[4][2][SC_BUF_BYTES];
+    __shared__ __attribute__((aligned(16))) float wsc_lds[NT > 1 ? 4 : 1][NT][LI_HEADS];
+    const int upb = (p.S1 + NT - 1) / NT;            // units per sequence
+    const int nunits = p.B * upb;
     const int w = threadIdx.x >> 6;
     const int l = threadIdx.x & 63;
     const int j = l & 31;
@@ -223,7 +242,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int tt = l + 64 * i;
-            int c = tt < p.T ? p.act[tt / p.S1] : 0;
+            int c = tt < nunits ? p.act[tt / upb] : 0;
             c = c < 0 ? 0 : (c > cap ? cap : c);
             pairs[i] = (c + 63) >> 6;
             total += pairs[i];
@@ -231,7 +250,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
         total = (int)wave_incl_scan((uint32_t)total);
         total = __builtin_amdgcn_readlane(total, 63);
         // every token may waste one run on rounding: plan for nwaves - T runs
-        ppw = (total + (nwaves - p.T) - 1) / (nwaves - p.T);
+        ppw = (total + (nwaves - nunits) - 1) / (nwaves - nunits);
         ppw = ppw < 1 ? 1 : (ppw > LI_MAX_PAIRS_PER_WAVE ? LI_MAX_PAIRS_PER_WAVE : ppw);
         int base = 0;                     // runs of all tokens before row i of the token table
         int found = -1;                   // token of this wave's run << 16 | run index... kept separately below
@@ -254,7 +273,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
         ppw = p.ppw;
         key0 = (blockIdx.x * 4 + w) * (ppw * 64);
     }
-    const int b = t / p.S1;
+    // t is the unit's number up to here; from here on its first token
+    const int b = t / upb;
+    const int s_first = (t - b * upb) * NT;
+    const int nt = p.S1 - s_first < NT ? p.S1 - s_first : NT;     // tokens of this unit (uniform)
+    t = b * p.S1 + s_first;
     int cur = p.act[b];
     cur = cur < 0 ? 0 : (cur > cap ? cap : cur);
     if (key0 >= cur) return;
@@ -319,19 +342,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
     // with the 32x32 accumulator layout (row = 8*(r/4) + 4*half + r%4) lane (key, half) then holds
     // heads 32*half + r in register r of accumulator 0 and heads 32*half + 16 + r in accumulator 1.
     // The contraction runs over 16-byte chunks in the order 4*half + ks (ks = 0..3).
-    i32x4 qa[2][4];
-    {
+    i32x4 qa[NT][2][4];
+#pragma unroll
+    for (int s = 0; s < NT; ++s) {
         const int head0 = 32 * ((j >> 2) & 1) + 4 * (j >> 3) + (j & 3);
-        const int8_t *q0 = p.q + ((size_t)t * LI_HEADS + head0) * LI_DIM + 64 * half;
+        const int ts = t + (s < nt ? s : 0);                   // a unit of one token loads that token twice
+        const int8_t *q0 = p.q + ((size_t)ts * LI_HEADS + head0) * LI_DIM + 64 * half;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            qa[0][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * ks);
-            qa[1][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * LI_DIM + 16 * ks);
+            qa[s][0][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * ks);
+            qa[s][1][ks] = *reinterpret_cast<const i32x4 *>(q0 + 16 * LI_DIM + 16 * ks);
         }
     }
-    // per-head factors: lane l computes head l's; read back lane by lane they are wave-uniform.
+    // per-head factors: lane l computes head l's.  One token per wave: read back lane by lane they are
+    // wave-uniform and sit in scalar registers.  Two tokens: they go to this wave's rows of wsc_lds and are
+    // read as broadcasts, four heads at a time, along the head sum.
     // VAR = 1 keeps the fp16 query scales and weights of head pairs (2i, 2i+1) packed instead.
-    float wsc[VAR ? 1 : LI_HEADS];
+    static_assert(!(VAR && NT > 1), "the fp16 variant scores one token per wave");
+    float wsc[(VAR || NT > 1) ? 1 : LI_HEADS];
     uint32_t qs2[VAR ? LI_HEADS / 2 : 1], w2[VAR ? LI_HEADS / 2 : 1];
     if (VAR) {
         const uint32_t mq = reinterpret_cast<const uint32_t *>(p.q_scale)[(size_t)t * (LI_HEADS / 2) + (l & 31)];
@@ -341,14 +369,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             qs2[h] = (uint32_t)__builtin_amdgcn_readlane((int)mq, h);
             w2[h] = (uint32_t)__builtin_amdgcn_readlane((int)mw, h);
         }
+    } else if (NT > 1) {
+#pragma unroll
+        for (int s = 0; s < NT; ++s) wsc_lds[w][s][l] = w_scale_of(p, (size_t)(t + (s < nt ? s : 0)) * LI_HEADS + l);
     } else {
         const float mine = w_scale_of(p, (size_t)t * LI_HEADS + l);
 #pragma unroll
         for (int h = 0; h < LI_HEADS; ++h) wsc[h] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, mine), h));
     }
 
-    float *srow = p.scores + (size_t)t * p.score_stride;
-    float *smp = p.sample + (size_t)t * (p.score_stride / LI_SAMPLE_GROUP);
+    float *srow0 = p.scores + (size_t)t * p.score_stride;
+    float *smp0 = p.sample + (size_t)t * (p.score_stride / LI_SAMPLE_GROUP);
     // 2^-11 as a run-time value, so that it sits in a scalar register (the mix instructions take no literal)
     const float scale = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3a000000));
     // this lane's operand chunks of row j inside a staged block
@@ -388,75 +419,97 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void l
             ksc = KDT == PTO_DT_BF16 ? bf16_bits_to_f32(hbits) : (float)__builtin_bit_cast(_Float16, hbits);
             ks2 = (uint32_t)hbits | ((uint32_t)hbits << 16);
         }
-        i32x16 ax0, ax1, ay0, ay1;
+        // the staged pair serves every token of the unit
+        auto score_token = [&](auto s_tag, float *srow, float *smp) {
+            constexpr int s = decltype(s_tag)::value;
+            i32x16 ax0, ax1, ay0, ay1;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { ax0[r] = 0; ax1[r] = 0; ay0[r] = 0; ay1[r] = 0; }
+            for (int r = 0; r < 16; ++r) { ax0[r] = 0; ax1[r] = 0; ay0[r] = 0; ay1[r] = 0; }
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            ax0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[0][ks], kx[ks], ax0, 0, 0, 0);
-            ax1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[1][ks], kx[ks], ax1, 0, 0, 0);
-            ay0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[0][ks], ky[ks], ay0, 0, 0, 0);
-            ay1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[1][ks], ky[ks], ay1, 0, 0, 0);
-        }
-        // lo[o][i] / hi[o][i]: heads 16*o + 2*i, +1 (lo) and 32 + 16*o + 2*i, +1 (hi) of this lane's key
-        uint32_t lo[2][8], hi[2][8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t x0 = VAR ? fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale) : relu_fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale);
-            const uint32_t y0 = VAR ? fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale) : relu_fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale);
-            const uint32_t x1 = VAR ? fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale) : relu_fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale);
-            const uint32_t y1 = VAR ? fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale) : relu_fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale);
-            const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
-            lo[0][i] = s0[0]; hi[0][i] = s0[1];
-            lo[1][i] = s1[0]; hi[1][i] = s1[1];
-        }
-        float sum = 0.f;
-        if (VAR) {
-            const float one = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3f800000));
-#pragma unroll
-            for (int o = 0; o < 2; ++o) {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint32_t v = dequant_relu_weight(lo[o][i], qs2[8 * o + i], ks2, w2[8 * o + i]);
-                    sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
-                    sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
-                }
+            for (int ks = 0; ks < 4; ++ks) {
+                ax0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[s][0][ks], kx[ks], ax0, 0, 0, 0);
+                ax1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[s][1][ks], kx[ks], ax1, 0, 0, 0);
+                ay0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[s][0][ks], ky[ks], ay0, 0, 0, 0);
+                ay1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa[s][1][ks], ky[ks], ay1, 0, 0, 0);
             }
+            // lo[o][i] / hi[o][i]: heads 16*o + 2*i, +1 (lo) and 32 + 16*o + 2*i, +1 (hi) of this lane's key
+            uint32_t lo[2][8], hi[2][8];
 #pragma unroll
-            for (int o = 0; o < 2; ++o) {
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t x0 = VAR ? fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale) : relu_fp16_pair(ax0[2 * i], ax0[2 * i + 1], scale);
+                const uint32_t y0 = VAR ? fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale) : relu_fp16_pair(ay0[2 * i], ay0[2 * i + 1], scale);
+                const uint32_t x1 = VAR ? fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale) : relu_fp16_pair(ax1[2 * i], ax1[2 * i + 1], scale);
+                const uint32_t y1 = VAR ? fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale) : relu_fp16_pair(ay1[2 * i], ay1[2 * i + 1], scale);
+                const auto s0 = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+                const auto s1 = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+                lo[0][i] = s0[0]; hi[0][i] = s0[1];
+                lo[1][i] = s1[0]; hi[1][i] = s1[1];
+            }
+            float sum = 0.f;
+            if (VAR) {
+                const float one = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(0x3f800000));
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint32_t v = dequant_relu_weight(hi[o][i], qs2[16 + 8 * o + i], ks2, w2[16 + 8 * o + i]);
-                    sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
-                    sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
+                for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t v = dequant_relu_weight(lo[o][i], qs2[8 * o + i], ks2, w2[8 * o + i]);
+                        sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
+                        sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
+                    }
+                }
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const uint32_t v = dequant_relu_weight(hi[o][i], qs2[16 + 8 * o + i], ks2, w2[16 + 8 * o + i]);
+                        sum = __fadd_rn(sum, mul_f16_f32<0>(v, one));
+                        sum = __fadd_rn(sum, mul_f16_f32<1>(v, one));
+                    }
+                }
+                const int pos = key0 + 64 * pr + l;
+                if (pos < cur) srow[pos] = sum;
+                if (sample_lane(pos, cur)) smp[pos >> 4] = sum;
+                return;
+            }
+            if (NT > 1) {
+                // heads ascending: lo[0][0..7], lo[1][0..7], hi[0][0..7], hi[1][0..7], two heads per register
+                const f32x4 *wrow = reinterpret_cast<const f32x4 *>(&wsc_lds[w][s][0]);
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    const f32x4 w4 = wrow[q];                        // heads 4q .. 4q+3, the same address on every lane
+                    const int o = (q >> 2) & 1, i = 2 * (q & 3);
+                    const uint32_t x0 = q < 8 ? lo[o][i] : hi[o][i], x1 = q < 8 ? lo[o][i + 1] : hi[o][i + 1];
+                    sum = __fadd_rn(sum, mul_f16_f32_v<0>(x0, w4[0]));
+                    sum = __fadd_rn(sum, mul_f16_f32_v<1>(x0, w4[1]));
+                    sum = __fadd_rn(sum, mul_f16_f32_v<0>(x1, w4[2]));
+                    sum = __fadd_rn(sum, mul_f16_f32_v<1>(x1, w4[3]));
+                }
+            } else {
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        sum = __fadd_rn(sum, mul_f16_f32<0>(lo[o][i], wsc[16 * o + 2 * i]));
+                        sum = __fadd_rn(sum, mul_f16_f32<1>(lo[o][i], wsc[16 * o + 2 * i + 1]));
+                    }
+                }
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        sum = __fadd_rn(sum, mul_f16_f32<0>(hi[o][i], wsc[32 + 16 * o + 2 * i]));
+                        sum = __fadd_rn(sum, mul_f16_f32<1>(hi[o][i], wsc[32 + 16 * o + 2 * i + 1]));
+                    }
                 }
             }
             const int pos = key0 + 64 * pr + l;
-            if (pos < cur) srow[pos] = sum;
-            if (sample_lane(pos, cur)) smp[pos >> 4] = sum;
-            return;
-        }
-#pragma unroll
-        for (int o = 0; o < 2; ++o) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                sum = __fadd_rn(sum, mul_f16_f32<0>(lo[o][i], wsc[16 * o + 2 * i]));
-                sum = __fadd_rn(sum, mul_f16_f32<1>(lo[o][i], wsc[16 * o + 2 * i + 1]));
-            }
-        }
-#pragma unroll
-        for (int o = 0; o < 2; ++o) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                sum = __fadd_rn(sum, mul_f16_f32<0>(hi[o][i], wsc[32 + 16 * o + 2 * i]));
-                sum = __fadd_rn(sum, mul_f16_f32<1>(hi[o][i], wsc[32 + 16 * o + 2 * i + 1]));
-            }
-        }
-        const int pos = key0 + 64 * pr + l;
-        const float sc = __fmul_rn(sum, ksc);
-        if (pos < cur) srow[pos] = sc;
-        if (sample_lane(pos, cur)) smp[pos >> 4] = sc;
+            const float sc = __fmul_rn(sum, ksc);
+            if (pos < cur) srow[pos] = sc;
+            if (sample_lane(pos, cur)) smp[pos >> 4] = sc;
+        };
+        score_token(std::integral_constant<int, 0>{}, srow0, smp0);
+        if (NT > 1 && nt > 1)
+            score_token(std::integral_constant<int, NT - 1>{}, srow0 + p.score_stride, smp0 + p.score_stride / LI_SAMPLE_GROUP);
     };
     for (int pr = 0; pr < npair; pr += 2) {
         trip(pr, 0);
@@ -1029,17 +1082,25 @@ __global__ __launch_bounds__(SEL_THREADS) void li_select_stream_kernel(const LiP
 hipError_t li_launch(const LiParams &p, hipStream_t stream)
 {
     const dim3 block(256);
+    const int nt = p.nt;
+    const int nunits = p.B * ((p.S1 + nt - 1) / nt);
     dim3 grid;
     if (p.balanced) {
         grid = dim3((unsigned)p.score_wgs);
     } else {
         const unsigned gx = (unsigned)((p.score_stride + 4 * p.ppw * 64 - 1) / (4 * p.ppw * 64));
-        grid = dim3(gx, (unsigned)p.T);
+        grid = dim3(gx, (unsigned)nunits);
     }
     if (p.variant == 1) hipLaunchKernelGGL((li_score_kernel<PTO_DT_FP16, 1>), grid, block, 0, stream, p);
-    else if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
-    else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP16>, grid, block, 0, stream, p);
-    else hipLaunchKernelGGL(li_score_kernel<PTO_DT_BF16>, grid, block, 0, stream, p);
+    else if (nt == 2) {
+        if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL((li_score_kernel<PTO_DT_FP32, 0, 2>), grid, block, 0, stream, p);
+        else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL((li_score_kernel<PTO_DT_FP16, 0, 2>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((li_score_kernel<PTO_DT_BF16, 0, 2>), grid, block, 0, stream, p);
+    } else {
+        if (p.k_dt == PTO_DT_FP32) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP32>, grid, block, 0, stream, p);
+        else if (p.k_dt == PTO_DT_FP16) hipLaunchKernelGGL(li_score_kernel<PTO_DT_FP16>, grid, block, 0, stream, p);
+        else hipLaunchKernelGGL(li_score_kernel<PTO_DT_BF16>, grid, block, 0, stream, p);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(li_select_kernel, dim3((unsigned)p.T), dim3(SEL_THREADS), 0, stream, p);

@@ -122,6 +122,19 @@ def test_many_query_tokens_short_sequences(c_oracle, b, s1):
     assert_exact(run_op(inp), oracle(inp, c_oracle), f"b={b} s1={s1}")
 
 
+@pytest.mark.parametrize("variant,b,s1", [("fp32", 28, 3), ("fp16", 28, 4)])
+def test_token_pairs_share_a_key_pass(c_oracle, variant, b, s1):
+    """Enough work for the launch to score two query tokens of a sequence per key pass (the reference scores
+    all s1 tokens against a page at once, lightning_indexer_quant_impl.py:163-169): an odd s1 leaves a unit of
+    one token, s1 = 4 makes two units per sequence; ragged lengths end inside runs and pairs."""
+    g = torch.Generator().manual_seed(300 + b)
+    act = [int(x) for x in torch.randint(2100, 20480, [b], generator=g)]
+    act[0], act[1] = 20480, 2049
+    inp = gen_indexer_inputs(b, s1, act, selected_count=2048, seed=b * s1, variant=variant)
+    assert inp.b * ((s1 + 1) // 2) * (inp.block_table.shape[1] * 128 // 64) >= 8 * 256 * 8, "shape too small for token pairs"
+    assert_exact(run_op(inp), oracle(inp, c_oracle), f"{variant} b={b} s1={s1}")
+
+
 def test_small_pages_and_small_k(c_oracle):
     """32-key pages (every block of a pair on its own page) and small selection counts."""
     for k, act in ((1, [5000, 70]), (17, [2500, 31]), (512, [700, 513])):
