@@ -12,8 +12,9 @@ timed region.  Prints ONE JSON line:
                  the HBM-side figure (algorithmic bytes / same duration, against 8 TB/s) is in
                  "roofline_hbm" because the shape sits at the ridge of the two
   packed_cache   the same step through sparse_attention_antiquant_d (one 656-byte row per key)
-  indexer        time of one lightning-indexer pass (score + select) on the same batch and on the
-                 indexer-only configuration (B=4, KV 32768), with its HBM fraction
+  indexer        time of one lightning-indexer pass (score + select) on the same batch, on the
+                 indexer-only configuration (B=4, KV 32768) and on configs[3]'s batch (B=64, two query
+                 tokens per sequence), with its HBM fraction and the counter-derived HBM traffic
   indexer_prolog time of one lightning-indexer prolog pass (projection stage) on the reference's enabled
                  case b=4, s1=2 (8 tokens, h=7168, q_lora_rank=1536), launches replayed from a HIP graph so
                  that host time between launches is not counted, with its HBM fraction
@@ -42,20 +43,33 @@ PEAK_HBM_GBS = 8000.0
 ROT = 8
 COPY_MIB = 256
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "sfa_decode_cfg2_hbm_traffic.md")
+LI_TRAFFIC_FILE = os.path.join(ROOT, "profiles", "indexer_hbm_traffic.md")
 
 
-def measured_traffic():
-    """HBM bytes per attention step from the committed counter runs (FETCH_SIZE and WRITE_SIZE of the
-    step's kernels, scaled by what the same counters read for a device copy of known size): the line
-    'traffic_bytes_per_step: N' of the summary under profiles/, or None."""
+def measured_traffic(path, key, library_version, expect=None):
+    """HBM bytes per launch from a committed counter summary under profiles/ (FETCH_SIZE and WRITE_SIZE of the
+    kernels, scaled by what the same counters read for a device copy of known size): the line '<key>: N'.
+    The summary names the library version it was taken with ('library_version: x.y.z') and may name other
+    launch facts ('<name>: value' lines listed in `expect`); when any of them no longer matches the built
+    library the figure is stale and None is returned instead."""
     try:
-        with open(TRAFFIC_FILE) as f:
+        fields = {}
+        with open(path) as f:
             for ln in f:
-                if ln.startswith("traffic_bytes_per_step:"):
-                    return int(ln.split(":")[1].strip())
+                m = ln.strip().split(":", 1)
+                if len(m) == 2 and " " not in m[0]:
+                    fields[m[0]] = m[1].strip()
     except OSError:
-        pass
-    return None
+        return None
+    if fields.get("library_version") != library_version or key not in fields:
+        return None
+    for name, want in (expect or {}).items():
+        if fields.get(name) != str(want):
+            return None
+    try:
+        return int(fields[key])
+    except ValueError:
+        return None
 
 
 def sfa_algorithmic_work(cur_seqs, n_heads=128):
@@ -88,6 +102,21 @@ def time_events(fn, steps, warmup, torch):
     wall = time.perf_counter() - t0
     per = [a.elapsed_time(b) for a, b in evs]            # ms, device time of the launches of one step
     return wall, sum(per) / len(per), min(per)
+
+
+def time_batch(fn, steps, warmup, torch):
+    """Average device time per step of `steps` back-to-back steps: one HIP event pair around the whole batch
+    (no host synchronisation and no event between the steps, as the steps of a decode loop follow one another)."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for i in range(steps):
+        fn(warmup + i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
 
 
 def prolog_leg(torch, dev, pypto_amd, b=4, s1=2, calls=20, replays=10):
@@ -334,6 +363,15 @@ def main():
     if args.counter_run:
         for i in range(2 * ROT):
             sfa_step(i)
+        # the indexer on the same batch and on configs[1], for its kernels' counters
+        res_c = torch.empty([B, 1, K], dtype=torch.int32, device=dev)
+        li1_c = gen_indexer_inputs(4, 1, config_lengths(1), selected_count=K, seed=1, variant="fp32").to(dev)
+        for i in range(ROT):
+            pypto_amd.lightning_indexer_decode(idx_queries[i], li_d.idx_query_scale, li_d.idx_key_cache, li_d.idx_key_scale,
+                                               li_d.idx_weight, li_d.act_seq_key, li_d.block_table, res_c, None, None, K)
+            pypto_amd.lightning_indexer_decode(li1_c.idx_query, li1_c.idx_query_scale, li1_c.idx_key_cache,
+                                               li1_c.idx_key_scale, li1_c.idx_weight, li1_c.act_seq_key, li1_c.block_table,
+                                               li1_c.topk_res, None, None, K)
         src = torch.empty(COPY_MIB << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
         dst.copy_(src)
@@ -355,6 +393,13 @@ def main():
 
     cur_seqs = [min(L, K) for L in lengths]
     byt, flops = sfa_algorithmic_work(cur_seqs, NQ)
+    # what the committed counter summaries must have been taken with to still describe this library
+    from pypto_amd import _native
+    C = _native.load()
+    lib_version = C.version()
+    ws_bytes = C.sfa_quant_workspace_bytes(B, S1, NQ, 1, K, 128, int(sfa_d.block_table.shape[1]), int(sfa_d.key_nope_2d.shape[0]),
+                                           float(sfa.softmax_scale), 0)
+    key_splits = max(ws_bytes // (B * S1 * NQ * (512 * 2 + 8)), 1)
     achieved_tflops = flops / (ev_avg_ms * 1e-3) / 1e12
     achieved_gbs = byt / (ev_avg_ms * 1e-3) / 1e9
 
@@ -381,7 +426,7 @@ def main():
         pypto_amd.lightning_indexer_decode(idx_queries[i % ROT], li_d.idx_query_scale, li_d.idx_key_cache,
                                            li_d.idx_key_scale, li_d.idx_weight, li_d.act_seq_key, li_d.block_table,
                                            res, None, None, K)
-    _, li2_avg_ms, _ = time_events(li_step, max(args.steps // 4, 5), 20, torch)
+    li2_avg_ms = time_batch(li_step, max(args.steps // 2, 40), 20, torch)
     li2_bytes = indexer_algorithmic_bytes(lengths, 4)
 
     li1 = gen_indexer_inputs(4, 1, config_lengths(1), selected_count=K, seed=1, variant="fp32").to(dev)
@@ -390,8 +435,22 @@ def main():
         pypto_amd.lightning_indexer_decode(li1.idx_query, li1.idx_query_scale, li1.idx_key_cache, li1.idx_key_scale,
                                            li1.idx_weight, li1.act_seq_key, li1.block_table, li1.topk_res, None, None,
                                            K)
-    _, li1_avg_ms, _ = time_events(li1_step, max(args.steps // 4, 5), 20, torch)
+    li1_avg_ms = time_batch(li1_step, max(args.steps // 2, 40), 20, torch)
     li1_bytes = indexer_algorithmic_bytes(config_lengths(1), 4)
+    del li1
+
+    # configs[3]'s indexer: B=64, two query tokens per sequence (the pair shares one pass over the keys)
+    len3 = config_lengths(3, seed=3)
+    li3 = gen_indexer_inputs(64, 2, len3, selected_count=K, seed=3, variant="fp32").to(dev)
+
+    def li3_step(i):
+        pypto_amd.lightning_indexer_decode(li3.idx_query, li3.idx_query_scale, li3.idx_key_cache, li3.idx_key_scale,
+                                           li3.idx_weight, li3.act_seq_key, li3.block_table, li3.topk_res, None, None,
+                                           K)
+    li3_avg_ms = time_batch(li3_step, max(args.steps // 4, 20), 10, torch)
+    # per sequence: the keys once, two tokens' queries, factors and results
+    li3_bytes = sum(L * (128 + 4) + 2 * (64 * 128 + 64 * 8 + K * 4) + 4 * math.ceil(L / 128) for L in len3)
+    del li3
 
     # ------------------------------------------------------------------ indexer prolog (projection stage)
     # the side legs must not cost the headline line: a failure there is reported in its field
@@ -443,7 +502,9 @@ def main():
                                f"shuffled block table, {ROT} rotating selections",
                    "kv_rows": int(sfa.key_nope_2d.shape[0]), "sum_kv_len": int(sum(lengths))},
         "roofline": {"bound": "mfma", "achieved": achieved_tflops, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved_tflops / PEAK_BF16_TFLOPS, "traffic": measured_traffic(),
+                     "frac": achieved_tflops / PEAK_BF16_TFLOPS,
+                     "traffic": measured_traffic(TRAFFIC_FILE, "traffic_bytes_per_step", lib_version,
+                                                 {"key_splits": key_splits}),
                      "kernel": "sfa_decode_kernel<4> + sfa_combine_kernel (one step)",
                      "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "flops_per_launch": flops},
         "roofline_hbm": {"bound": "hbm", "achieved": achieved_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -452,7 +513,12 @@ def main():
                          "bit_identical_to_three_array_result": packed_same},
         "indexer": {"configs[2]_us_per_step": li2_avg_ms * 1e3, "configs[2]_hbm_frac": li2_bytes / (li2_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
                     "configs[1]_us_per_step": li1_avg_ms * 1e3, "configs[1]_hbm_frac": li1_bytes / (li1_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS,
-                    "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes, "scale_dtype": "fp32", "weight_dtype": "bf16"},
+                    "bytes_configs[2]": li2_bytes, "bytes_configs[1]": li1_bytes,
+                    "traffic_configs[2]": measured_traffic(LI_TRAFFIC_FILE, "indexer_traffic_bytes_configs2", lib_version),
+                    "traffic_configs[1]": measured_traffic(LI_TRAFFIC_FILE, "indexer_traffic_bytes_configs1", lib_version),
+                    "configs[3]_us_per_step": li3_avg_ms * 1e3,
+                    "configs[3]_hbm_frac": li3_bytes / (li3_avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, "bytes_configs[3]": li3_bytes,
+                    "scale_dtype": "fp32", "weight_dtype": "bf16"},
         "indexer_prolog": prolog,
         "mla_prolog": mla_prolog,
         "mla_indexer_prolog": fused_prolog,
