@@ -371,6 +371,12 @@ typedef struct PtoMlaPrologQuantArgs {
     int64_t cache_rows;   /* block_num * block_size */
     float epsilon_cq;
     float epsilon_ckv;
+    int32_t absorb_exact; /* query_nope = (query . w_uk): 1 = fixed-order fp32 sums (bit-reproducible, the statement
+                             above); 0 = on the matrix cores: the same exact bf16 products summed in fp32 in the
+                             cores' order, so some results differ in the last bf16 bit -- inside the reference's
+                             own acceptance rule for this output (deepseekv32_mla_prolog_quant.py:668-692), which
+                             only feeds the attention.  Every other output is the same either way. */
+    int32_t reserved;
 } PtoMlaPrologQuantArgs;
 
 int pto_mla_prolog_quant_workspace_bytes(const PtoMlaPrologQuantArgs *args, size_t *bytes);

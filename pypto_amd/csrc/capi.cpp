@@ -617,6 +617,7 @@ int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream
     p.n_heads = (int)a->n_heads;
     p.eps_cq = a->epsilon_cq;
     p.eps_ckv = a->epsilon_ckv;
+    p.absorb_exact = a->absorb_exact ? 1 : 0;
     hipError_t e = pto::mlap_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;

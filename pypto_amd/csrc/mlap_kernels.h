@@ -40,6 +40,9 @@ struct MlapParams {
     long long cache_rows;
     int T, h, q_lora, n_heads;
     float eps_cq, eps_ckv;
+    int absorb_exact;             // 1: the product with w_uk as fixed-order fp32 sums (bit-reproducible against the
+                                  // sequential statement); 0: on the matrix cores (bf16 x bf16 exact, fp32 sums in the
+                                  // cores' own order: differs in the last bit of some results)
 };
 
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);

@@ -271,6 +271,7 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
 {
     __shared__ __attribute__((aligned(16))) uint8_t wsl[4 * FIN_W_BYTES];
     __shared__ __attribute__((aligned(16))) float arow[MLAP_XTOK][MLAP_NOPE];
+    __shared__ __attribute__((aligned(16))) uint16_t abf[MLAP_XTOK][MLAP_NOPE];      // the same values as bf16 (they are bf16-valued)
     const int l = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int head = blockIdx.x % p.n_heads;
@@ -307,6 +308,7 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
             f32x2 av = {bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0])),
                         bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]))};
             *reinterpret_cast<f32x2 *>(&arow[tl][2 * l]) = av;
+            *reinterpret_cast<uint32_t *>(&abf[tl][2 * l]) = pack_bf16x2(av[0], av[1]);
         }
         // rope part (first half-workgroup only): lane l < 32 -> channels 2l, 2l+1 = rotation partners l, 32+l
         if (half == 0 && l < 32 && t < p.T) {
@@ -333,6 +335,47 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
     VM_WAIT(0);
     __syncthreads();
 
+    if (!p.absorb_exact) {
+        // On the matrix cores: C^T[col][token] = sum_i W^T[col][i] a^T[i][token], v_mfma_f32_32x32x16_bf16 with
+        // A = the wave's slice of w_uk read transposed out of LDS (ds_read_b64_tr_b16: lane (col, half) gets rows
+        // 16ks + 4*half + 0..3 and 16ks + 8 + 4*half + 0..3 of its column), B = the tokens' query values in the same
+        // row order (lanes of tokens 8..31 repeat token 0; their results are not stored).  Two blocks of 32
+        // columns, eight contraction steps.  Lane (token, half) then holds columns 8*(r/4) + 4*half + r%4 of a block.
+        const uint16_t *wt = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) +
+                             (4 * (l >> 5) + ((l & 15) >> 2)) * 64 + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+        const int tok = (l & 31) < MLAP_XTOK ? (l & 31) : 0;
+        const uint16_t *at = &abf[tok][4 * (l >> 5)];
+        f32x16 c[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c[cb][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < MLAP_NOPE / 16; ++ks) {
+            const u32x2 b0 = *reinterpret_cast<const u32x2 *>(at + 16 * ks);
+            const u32x2 b1 = *reinterpret_cast<const u32x2 *>(at + 16 * ks + 8);
+            const u32x4 bq = {b0[0], b0[1], b1[0], b1[1]};
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) {
+                const s16x4 a0 = lds_read_tr16(wt + (16 * ks) * 64 + 32 * cb);
+                const s16x4 a1 = lds_read_tr16(wt + (16 * ks + 8) * 64 + 32 * cb);
+                const s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+                c[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, bq), c[cb], 0, 0, 0);
+            }
+        }
+        const int t = t0 + (l & 31);
+        if ((l & 31) < MLAP_XTOK && t < p.T) {
+            uint16_t *dst = p.q_nope + ((size_t)t * p.n_heads + head) * MLAP_KV + colbase + 4 * (l >> 5);
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const u32x2 v = {pack_bf16x2(c[cb][4 * q], c[cb][4 * q + 1]), pack_bf16x2(c[cb][4 * q + 2], c[cb][4 * q + 3])};
+                    *reinterpret_cast<u32x2 *>(dst + 32 * cb + 8 * q) = v;
+                }
+        }
+        return;
+    }
     // out[t][colbase + 64w + l] = sum_i a[t][i] * w_uk[head][i][col], i ascending; 8 tokens at once.
     // Chunks of four rows are read one chunk ahead of the multiply-adds that consume them.
     const uint16_t *wl = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) + l;

@@ -254,7 +254,7 @@ PYBIND11_MODULE(_C, m)
              std::uintptr_t q_norm_out, std::uintptr_t q_norm_scale_out, std::uintptr_t query_nope_out,
              std::uintptr_t query_rope_out, std::uintptr_t workspace, size_t workspace_bytes, int64_t t, int64_t h,
              int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows, double epsilon_cq, double epsilon_ckv,
-             std::uintptr_t stream) {
+             bool absorb_exact, std::uintptr_t stream) {
               PtoMlaPrologQuantArgs a{};
               a.token_x = ptr<const void>(token_x);
               a.w_dq = ptr<const void>(w_dq);
@@ -283,6 +283,7 @@ PYBIND11_MODULE(_C, m)
               a.cache_rows = cache_rows;
               a.epsilon_cq = static_cast<float>(epsilon_cq);
               a.epsilon_ckv = static_cast<float>(epsilon_ckv);
+              a.absorb_exact = absorb_exact ? 1 : 0;
               check(pto_mla_prolog_quant_launch(&a, ptr<void>(stream)));
           });
 }

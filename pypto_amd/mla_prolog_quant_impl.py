@@ -14,6 +14,12 @@ Outputs are pre-allocated by the caller and written in place: ``q_norm_out``, ``
 ``query_nope_out``, ``query_rope_out`` and rows ``cache_index[i]`` of the three caches (the ``*_out`` cache
 arguments normally alias the inputs, as in the reference driver :576-577, 616-617; when they do not, the cache
 is copied first).  Returns ``None``; runs asynchronously on the current stream.
+
+``EXACT_ABSORB`` (module attribute, default ``False``) chooses how ``query_nope = query . w_uk`` is summed: on the
+matrix cores (the default: the same exact bf16 products, fp32 sums in the cores' order, so some results differ in
+the last bf16 bit from the sequential statement -- inside the reference's own acceptance rule for this output,
+deepseekv32_mla_prolog_quant.py:668-692) or, when ``True``, as fixed-order fp32 sums that reproduce the
+sequential statement bit for bit.  Every other output is the same either way.
 """
 from __future__ import annotations
 
@@ -24,6 +30,9 @@ import torch
 
 from . import _native
 from .converter import as_torch
+
+
+EXACT_ABSORB = False
 
 
 class MlaTileConfig:
@@ -147,7 +156,8 @@ def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gam
                                   wdkv.data_ptr(), gcq.data_ptr(), gckv.data_ptr(), cs.data_ptr(), sn.data_ptr(),
                                   cidx.data_ptr(), kvc.data_ptr(), krc.data_ptr(), ksc.data_ptr(), qn.data_ptr(),
                                   qns.data_ptr(), qnope.data_ptr(), qrope.data_ptr(), ws.data_ptr(), ws_bytes, t, h,
-                                  q_lora, n_heads, cache_rows, float(epsilon_cq), float(epsilon_ckv), stream)
+                                  q_lora, n_heads, cache_rows, float(epsilon_cq), float(epsilon_ckv), bool(EXACT_ABSORB),
+                                  stream)
     return None
 
 
