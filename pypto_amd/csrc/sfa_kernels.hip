@@ -707,22 +707,41 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                 for (int b4 = 0; b4 < 4; ++b4)
 #pragma unroll
                     for (int q4 = 0; q4 < 4; ++q4) {
+                        // the accumulators leave their registers here and nowhere earlier
                         const f32x16 &acc = o[4 * gq + b4];
-                        const float v0 = acc[4 * q4] * inv, v1 = acc[4 * q4 + 1] * inv;
-                        const float v2 = acc[4 * q4 + 2] * inv, v3 = acc[4 * q4 + 3] * inv;
+                        float r0, r1, r2, r3;
+                        asm volatile("v_accvgpr_read_b32 %0, %4\n\tv_accvgpr_read_b32 %1, %5\n\tv_accvgpr_read_b32 %2, %6\n\tv_accvgpr_read_b32 %3, %7"
+                                     : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+                                     : "a"(acc[4 * q4]), "a"(acc[4 * q4 + 1]), "a"(acc[4 * q4 + 2]), "a"(acc[4 * q4 + 3]));
+                        const float v0 = r0 * inv, v1 = r1 * inv, v2 = r2 * inv, v3 = r3 * inv;
                         u32x2 pk;
                         pk[0] = FINAL ? pack_bf16x2(v0, v1) : pack_f16x2(v0, v1);
                         pk[1] = FINAL ? pack_bf16x2(v2, v3) : pack_f16x2(v2, v3);
                         *reinterpret_cast<u32x2 *>(stage + col * 256 + 8 * ((8 * b4 + 2 * q4 + half) ^ col)) = pk;
                     }
-#pragma unroll 2
-                for (int e = 0; e < 8; ++e) {
-                    const int hl = 4 * e + hsub;
-                    const u32x2 lo = *reinterpret_cast<const u32x2 *>(stage + hl * 256 + 8 * ((2 * j) ^ hl));
-                    const u32x2 hi = *reinterpret_cast<const u32x2 *>(stage + hl * 256 + 8 * ((2 * j + 1) ^ hl));
-                    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
-                    if (ALL || head_base + hl < p.NQ)
-                        *reinterpret_cast<u32x4 *>(dst0 + (size_t)(4 * e) * DN + 128 * gq) = v;
+                // Eight reads go out before the first store waits for its pair: written as assembly, because
+                // the compiler pairs every two reads with a wait of their own (eight exposed LDS latencies
+                // per chunk instead of two).
+#pragma unroll
+                for (int e0 = 0; e0 < 8; e0 += 4) {
+                    u32x2 lo[4], hi[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int hl = 4 * (e0 + e) + hsub;
+                        const uint32_t a_lo = (uint32_t)(uintptr_t)(lds_byte_t *)(stage + hl * 256 + 8 * ((2 * j) ^ hl));
+                        const uint32_t a_hi = (uint32_t)(uintptr_t)(lds_byte_t *)(stage + hl * 256 + 8 * ((2 * j + 1) ^ hl));
+                        asm volatile("ds_read_b64 %0, %1" : "=v"(lo[e]) : "v"(a_lo) : "memory");
+                        asm volatile("ds_read_b64 %0, %1" : "=v"(hi[e]) : "v"(a_hi) : "memory");
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int hl = 4 * (e0 + e) + hsub;
+                        asm volatile("" : "+v"(lo[e]), "+v"(hi[e]));
+                        const u32x4 v = {lo[e][0], lo[e][1], hi[e][0], hi[e][1]};
+                        if (ALL || head_base + hl < p.NQ)
+                            *reinterpret_cast<u32x4 *>(dst0 + (size_t)(4 * (e0 + e)) * DN + 128 * gq) = v;
+                    }
                 }
             }
         };
