@@ -69,3 +69,18 @@ def as_torch(x, what: str) -> torch.Tensor:
             raise RuntimeError(f"{what}: not all tensors are contiguous")
         return x
     raise TypeError(f"{what}: input type is not currently supported.")
+
+
+def copy_unless_same(dst: torch.Tensor, src: torch.Tensor, what: str) -> None:
+    """The cache-out arguments of the prolog operators: normally the very tensor passed as cache-in (the
+    kernels then update the rows named by the cache index in place and nothing is copied).  A different
+    tensor receives a copy of the whole cache first -- the reference's semantics, and gigabytes per call at
+    real cache sizes, so in-place use is the intended path.  Two views that share memory without being the
+    same range would be copied onto themselves: refused."""
+    if dst.data_ptr() == src.data_ptr():
+        return
+    lo_d, lo_s = dst.data_ptr(), src.data_ptr()
+    hi_d, hi_s = lo_d + dst.numel() * dst.element_size(), lo_s + src.numel() * src.element_size()
+    if lo_d < hi_s and lo_s < hi_d:
+        raise ValueError(f"{what} and {what}_out overlap in memory without being the same tensor")
+    dst.copy_(src.reshape(dst.shape))

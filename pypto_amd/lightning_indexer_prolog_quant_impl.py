@@ -24,7 +24,7 @@ from typing import List, Optional
 import torch
 
 from . import _native
-from .converter import as_torch
+from .converter import as_torch, copy_unless_same
 
 
 @dataclass
@@ -151,10 +151,8 @@ def lightning_indexer_prolog_quant(x_in, q_norm_in, q_norm_scale_in, w_qb_in, w_
         raise ValueError("w_qb must be (q_lora_rank, n_heads*128) and wk (h, 128)")
     if kc_in.shape != kc.shape or ks_in.numel() != ks.numel():
         raise ValueError("k_int8_in/k_scale_in and k_int8_out/k_scale_out differ in shape")
-    if kc.data_ptr() != kc_in.data_ptr():
-        kc.copy_(kc_in)
-    if ks.data_ptr() != ks_in.data_ptr():
-        ks.copy_(ks_in.reshape(ks.shape))
+    copy_unless_same(kc, kc_in, "k_int8")
+    copy_unless_same(ks, ks_in, "k_scale")
 
     ws_bytes = C.li_prolog_quant_workspace_bytes(t, h, q_lora, n_heads, cache_rows)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)

@@ -29,7 +29,7 @@ from typing import List, Optional
 import torch
 
 from . import _native
-from .converter import as_torch
+from .converter import as_torch, copy_unless_same
 
 
 EXACT_ABSORB = False
@@ -145,8 +145,7 @@ def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gam
     for a, b_, nm in ((kvc, kvc_in, "kv_cache"), (krc, krc_in, "kr_cache"), (ksc, ksc_in, "k_scale_cache")):
         if a.numel() != b_.numel() or a.dtype != b_.dtype:
             raise ValueError(f"{nm} and {nm}_out differ in shape or type")
-        if a.data_ptr() != b_.data_ptr():
-            a.copy_(b_.reshape(a.shape))
+        copy_unless_same(a, b_, nm)
 
     ws_bytes = C.mla_prolog_quant_workspace_bytes(t, h, q_lora, n_heads, cache_rows)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)

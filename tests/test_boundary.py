@@ -126,3 +126,17 @@ def test_prolog_operators_refuse_cpu_tensors_and_unbuilt_variants():
     args[3] = None                                       # no dequant scale: the non-quantized up-projection
     with pytest.raises(ValueError):
         pypto_amd.mla_prolog_quant_d(*args, *mouts, 1e-5, 1e-5, "PA_BSND", None, None)
+
+
+def test_cache_out_overlapping_cache_in_is_refused():
+    """The prolog operators copy cache-in to cache-out unless they are the same tensor; two views that share
+    memory without being the same range must not be copied onto each other."""
+    import torch
+    from pypto_amd.converter import copy_unless_same
+    base = torch.arange(64, dtype=torch.int8)
+    copy_unless_same(base[:32], base[:32], "k_int8")                 # same range: nothing happens
+    other = torch.zeros(32, dtype=torch.int8)
+    copy_unless_same(other, base[:32], "k_int8")                     # disjoint: copied
+    assert torch.equal(other, base[:32])
+    with pytest.raises(ValueError, match="overlap"):
+        copy_unless_same(base[8:40], base[:32], "k_int8")
