@@ -154,26 +154,47 @@ __global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapPara
     const bool active = w < nslab || rope_wave;
     const int col = (kvtype ? p.q_lora : 0) + w * 128 + 2 * (rope_wave ? (l & 31) : l);
 
+    // Everything the chain below needs from memory is requested before the first value is looked at: the
+    // cache row, the norm weights, the rotation factors and the group sums, sixteen groups at a time
+    // (taken one after the other, the fourteen group loads of a 7168-wide hidden axis alone were fourteen
+    // memory latencies).
+    const long long dst = kvtype ? p.cache_index[t] : -1;
+    uint32_t gm = 0;
+    if (w < nslab) gm = reinterpret_cast<const uint32_t *>(kvtype ? p.gamma_ckv : p.gamma_cq)[w * 64 + l];
+    uint16_t cs0 = 0, cs1 = 0, sn0 = 0, sn1 = 0;
+    if (rope_wave && l < 32) {
+        cs0 = p.cos[(size_t)t * MLAP_ROPE + l];
+        cs1 = p.cos[(size_t)t * MLAP_ROPE + 32 + l];
+        sn0 = p.sin[(size_t)t * MLAP_ROPE + l];
+        sn1 = p.sin[(size_t)t * MLAP_ROPE + 32 + l];
+    }
     float v0 = 0.f, v1 = 0.f;
     if (active) {
         const float *src = p.xpart + (size_t)t * nc + col;
-        for (int g = 0; g < ngroups; ++g) {
-            const f32x2 v = *reinterpret_cast<const f32x2 *>(src + (size_t)g * p.T * nc);
-            v0 = __fadd_rn(v0, v[0]);
-            v1 = __fadd_rn(v1, v[1]);
+        for (int g0 = 0; g0 < ngroups; g0 += 16) {
+            f32x2 v[16];
+#pragma unroll
+            for (int g = 0; g < 16; ++g)
+                v[g] = *reinterpret_cast<const f32x2 *>(src + (size_t)(g0 + g < ngroups ? g0 + g : ngroups - 1) * p.T * nc);
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                if (g0 + g < ngroups) {
+                    v0 = __fadd_rn(v0, v[g][0]);
+                    v1 = __fadd_rn(v1, v[g][1]);
+                }
+            }
         }
         v0 = bf16_round_f32(v0);
         v1 = bf16_round_f32(v1);
     }
-    const long long dst = kvtype ? p.cache_index[t] : -1;
     const bool dst_ok = dst >= 0 && dst < p.cache_rows;
 
     if (rope_wave) {
         // lane l < 32 holds channels 2l and 2l+1, which after the de-interleave are channels l and 32+l:
         // the two partners of one rotation
         if (l < 32) {
-            const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
-            const float s0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), s1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
+            const float c0 = bf16_bits_to_f32(cs0), c1 = bf16_bits_to_f32(cs1);
+            const float s0 = bf16_bits_to_f32(sn0), s1 = bf16_bits_to_f32(sn1);
             const float r0 = __builtin_fmaf(v0, c0, (-v1) * s0);      // products exact: one rounding
             const float r1 = __builtin_fmaf(v1, c1, v0 * s1);
             if (dst_ok) {
@@ -193,7 +214,6 @@ __global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapPara
         float s = 0.f;
         for (int j = 0; j < nslab; ++j) s = __fadd_rn(s, slabsum[j]);
         const float d = __builtin_sqrtf(__fadd_rn(s, kvtype ? p.eps_ckv : p.eps_cq));   // correctly rounded (__fsqrt_rn is the 1-ulp hardware root here)
-        const uint32_t gm = reinterpret_cast<const uint32_t *>(kvtype ? p.gamma_ckv : p.gamma_cq)[w * 64 + l];
         y0 = bf16_round_f32(__fmul_rn(__fdiv_rn(v0, d), __uint_as_float(gm << 16)));
         y1 = bf16_round_f32(__fmul_rn(__fdiv_rn(v1, d), __uint_as_float(gm & 0xffff0000u)));
         const float m = wave_max_f32(fmaxf(fabsf(y0), fabsf(y1)));
