@@ -382,6 +382,33 @@ typedef struct PtoMlaPrologQuantArgs {
 int pto_mla_prolog_quant_workspace_bytes(const PtoMlaPrologQuantArgs *args, size_t *bytes);
 int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *args, void *hip_stream);
 
+/*
+ * MLA prolog + lightning-indexer prolog as one operator (mla_indexer_prolog_quant_d/_p,
+ * examples/models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:49-138, 141-256 in the
+ * reference): the MLA prolog runs first; its int8 normalised query latent and that latent's
+ * scale -- intermediates the reference's caller never sees (:218-219) -- feed the indexer
+ * prolog; hidden states, rope tables and cache index are shared.
+ *
+ *   mla      as for pto_mla_prolog_quant_launch.  q_norm_out / q_norm_scale_out may be NULL:
+ *            the two intermediates then live in the common workspace.  workspace and
+ *            workspace_bytes of this part are ignored.
+ *   indexer  as for pto_li_prolog_quant_launch, of which x, q_norm, q_norm_scale,
+ *            cos_idx_rope, sin_idx_rope, k_cache_index, t, h, q_lora_rank, workspace and
+ *            workspace_bytes are ignored: taken from the MLA part and the common workspace.
+ *   workspace  pto_mla_indexer_prolog_quant_workspace_bytes() bytes, 256-byte aligned: the
+ *            intermediates and one area that serves the partial sums of both halves in turn.
+ * Six kernels on the given stream, nothing else; errors as for the two operators.
+ */
+typedef struct PtoMlaIndexerPrologQuantArgs {
+    PtoMlaPrologQuantArgs mla;
+    PtoLiPrologQuantArgs indexer;
+    void *workspace;
+    size_t workspace_bytes;
+} PtoMlaIndexerPrologQuantArgs;
+
+int pto_mla_indexer_prolog_quant_workspace_bytes(const PtoMlaIndexerPrologQuantArgs *args, size_t *bytes);
+int pto_mla_indexer_prolog_quant_launch(const PtoMlaIndexerPrologQuantArgs *args, void *hip_stream);
+
 /* Thread-local description of the last error on this thread ("" if none). */
 const char *pto_last_error(void);
 

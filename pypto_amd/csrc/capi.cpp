@@ -331,7 +331,7 @@ extern "C" {
 
 const char *pto_last_error(void) { return g_err; }
 
-const char *pto_version(void) { return "0.2.0"; }
+const char *pto_version(void) { return "0.3.0"; }
 
 int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
 {
@@ -621,6 +621,84 @@ int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream
     hipError_t e = pto::mlap_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
+}
+
+// ---- both prologs as one operator: the query latent and its scale live in the common workspace
+
+namespace {
+
+struct FusedPlan {
+    size_t q_norm_off, q_norm_scale_off, rest_off, total;
+    PtoMlaPrologQuantArgs mla;
+    PtoLiPrologQuantArgs idx;
+};
+
+// fills in what the two halves share and where the intermediates go (workspace base may be null: sizes only)
+int fused_plan(const PtoMlaIndexerPrologQuantArgs *a, FusedPlan *pl)
+{
+    if (!a) return fail(PTO_E_INVALID_ARG, "mla_indexer_prolog: args is NULL");
+    pl->mla = a->mla;
+    pl->idx = a->indexer;
+    pl->idx.x = a->mla.token_x;
+    pl->idx.cos_idx_rope = a->mla.cos;
+    pl->idx.sin_idx_rope = a->mla.sin;
+    pl->idx.k_cache_index = a->mla.cache_index;
+    pl->idx.t = a->mla.t;
+    pl->idx.h = a->mla.h;
+    pl->idx.q_lora_rank = a->mla.q_lora_rank;
+    int rc = mlap_check(&pl->mla);
+    if (rc != PTO_OK) return rc;
+    rc = lip_check(&pl->idx);
+    if (rc != PTO_OK) return rc;
+    const size_t qn = ((size_t)a->mla.t * a->mla.q_lora_rank + 255) & ~(size_t)255;
+    const size_t qs = ((size_t)a->mla.t * sizeof(float) + 255) & ~(size_t)255;
+    const size_t w_mla = mlap_ws_bytes(&pl->mla), w_idx = lip_ws_bytes(&pl->idx);
+    pl->q_norm_off = 0;
+    pl->q_norm_scale_off = qn;
+    pl->rest_off = qn + qs;
+    // the MLA prolog's partial sums are dead when the indexer prolog's kernels start: one area serves both
+    pl->total = qn + qs + (w_mla > w_idx ? w_mla : w_idx);
+    char *base = static_cast<char *>(a->workspace);
+    if (base) {
+        int8_t *q_norm = a->mla.q_norm_out ? a->mla.q_norm_out : reinterpret_cast<int8_t *>(base + pl->q_norm_off);
+        float *q_norm_scale = a->mla.q_norm_scale_out ? a->mla.q_norm_scale_out : reinterpret_cast<float *>(base + pl->q_norm_scale_off);
+        pl->mla.q_norm_out = q_norm;
+        pl->mla.q_norm_scale_out = q_norm_scale;
+        pl->idx.q_norm = q_norm;
+        pl->idx.q_norm_scale = q_norm_scale;
+        pl->mla.workspace = base + pl->rest_off;
+        pl->mla.workspace_bytes = w_mla;
+        pl->idx.workspace = base + pl->rest_off;
+        pl->idx.workspace_bytes = w_idx;
+    }
+    return PTO_OK;
+}
+
+}  // namespace
+
+int pto_mla_indexer_prolog_quant_workspace_bytes(const PtoMlaIndexerPrologQuantArgs *a, size_t *bytes)
+{
+    if (!bytes) return fail(PTO_E_INVALID_ARG, "mla_indexer_prolog: bytes is NULL");
+    FusedPlan pl;
+    int rc = fused_plan(a, &pl);
+    if (rc != PTO_OK) return rc;
+    *bytes = pl.total;
+    return PTO_OK;
+}
+
+int pto_mla_indexer_prolog_quant_launch(const PtoMlaIndexerPrologQuantArgs *a, void *hip_stream)
+{
+    FusedPlan pl;
+    int rc = fused_plan(a, &pl);
+    if (rc != PTO_OK) return rc;
+    if (!a->workspace || a->workspace_bytes < pl.total)
+        return fail(PTO_E_WORKSPACE, "mla_indexer_prolog: workspace of %zu bytes required, %zu given", pl.total,
+                    a->workspace ? a->workspace_bytes : (size_t)0);
+    if (reinterpret_cast<uintptr_t>(a->workspace) & 255)
+        return fail(PTO_E_INVALID_ARG, "mla_indexer_prolog: the workspace must be 256-byte aligned");
+    rc = pto_mla_prolog_quant_launch(&pl.mla, hip_stream);
+    if (rc != PTO_OK) return rc;
+    return pto_li_prolog_quant_launch(&pl.idx, hip_stream);
 }
 
 }  // extern "C"

@@ -2,6 +2,10 @@
 // HIP stream as an integer handle; no torch types appear here.  Argument errors raise ValueError,
 // everything else RuntimeError, carrying the library's own message.
 #include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <stdexcept>
+#include <vector>
 
 #include <cstdint>
 #include <stdexcept>
@@ -285,5 +289,81 @@ PYBIND11_MODULE(_C, m)
               a.epsilon_ckv = static_cast<float>(epsilon_ckv);
               a.absorb_exact = absorb_exact ? 1 : 0;
               check(pto_mla_prolog_quant_launch(&a, ptr<void>(stream)));
+          });
+
+    // both prologs as one operator: the pointers of each half in the order of its own launch function
+    // (18 of the MLA prolog up to query_rope_out, 19 of the indexer prolog up to weights; the ones the
+    // fused entry point ignores may be 0)
+    auto fused_args = [](const std::vector<std::uintptr_t> &m, const std::vector<std::uintptr_t> &x, std::uintptr_t workspace,
+                         size_t workspace_bytes, int64_t t, int64_t h, int64_t q_lora_rank, int64_t mla_heads,
+                         int64_t mla_cache_rows, double epsilon_cq, double epsilon_ckv, bool absorb_exact, int64_t idx_heads,
+                         int64_t idx_cache_rows, double idx_eps) {
+        if (m.size() != 18 || x.size() != 19) throw std::invalid_argument("mla_indexer_prolog: 18 + 19 pointers expected");
+        PtoMlaIndexerPrologQuantArgs a{};
+        a.mla.token_x = ptr<const void>(m[0]);
+        a.mla.w_dq = ptr<const void>(m[1]);
+        a.mla.w_uq_qr = ptr<const int8_t>(m[2]);
+        a.mla.dequant_scale = ptr<const float>(m[3]);
+        a.mla.w_uk = ptr<const void>(m[4]);
+        a.mla.w_dkv_kr = ptr<const void>(m[5]);
+        a.mla.gamma_cq = ptr<const void>(m[6]);
+        a.mla.gamma_ckv = ptr<const void>(m[7]);
+        a.mla.cos = ptr<const void>(m[8]);
+        a.mla.sin = ptr<const void>(m[9]);
+        a.mla.cache_index = ptr<const int64_t>(m[10]);
+        a.mla.kv_cache = ptr<int8_t>(m[11]);
+        a.mla.kr_cache = ptr<void>(m[12]);
+        a.mla.k_scale_cache = ptr<float>(m[13]);
+        a.mla.q_norm_out = ptr<int8_t>(m[14]);
+        a.mla.q_norm_scale_out = ptr<float>(m[15]);
+        a.mla.query_nope_out = ptr<void>(m[16]);
+        a.mla.query_rope_out = ptr<void>(m[17]);
+        a.mla.t = t;
+        a.mla.h = h;
+        a.mla.q_lora_rank = q_lora_rank;
+        a.mla.n_heads = mla_heads;
+        a.mla.cache_rows = mla_cache_rows;
+        a.mla.epsilon_cq = static_cast<float>(epsilon_cq);
+        a.mla.epsilon_ckv = static_cast<float>(epsilon_ckv);
+        a.mla.absorb_exact = absorb_exact ? 1 : 0;
+        a.indexer.w_qb = ptr<const int8_t>(x[3]);
+        a.indexer.w_qb_scale = ptr<const float>(x[4]);
+        a.indexer.wk = ptr<const void>(x[5]);
+        a.indexer.w_proj = ptr<const void>(x[6]);
+        a.indexer.ln_gamma_k = ptr<const void>(x[7]);
+        a.indexer.ln_beta_k = ptr<const void>(x[8]);
+        a.indexer.hadamard_q = ptr<const void>(x[11]);
+        a.indexer.hadamard_k = ptr<const void>(x[12]);
+        a.indexer.k_cache = ptr<int8_t>(x[13]);
+        a.indexer.k_cache_scale = ptr<void>(x[14]);
+        a.indexer.q_int8 = ptr<int8_t>(x[16]);
+        a.indexer.q_scale = ptr<void>(x[17]);
+        a.indexer.weights = ptr<void>(x[18]);
+        a.indexer.n_heads = idx_heads;
+        a.indexer.cache_rows = idx_cache_rows;
+        a.indexer.eps = static_cast<float>(idx_eps);
+        a.workspace = ptr<void>(workspace);
+        a.workspace_bytes = workspace_bytes;
+        return a;
+    };
+    m.def("mla_indexer_prolog_quant_workspace_bytes",
+          [fused_args](int64_t t, int64_t h, int64_t q_lora_rank, int64_t mla_heads, int64_t mla_cache_rows, int64_t idx_heads,
+                       int64_t idx_cache_rows) {
+              const std::vector<std::uintptr_t> m18(18, 0), x19(19, 0);
+              PtoMlaIndexerPrologQuantArgs a = fused_args(m18, x19, 0, 0, t, h, q_lora_rank, mla_heads, mla_cache_rows, 0.0, 0.0,
+                                                          false, idx_heads, idx_cache_rows, 0.0);
+              size_t bytes = 0;
+              check(pto_mla_indexer_prolog_quant_workspace_bytes(&a, &bytes));
+              return bytes;
+          });
+    m.def("mla_indexer_prolog_quant_launch",
+          [fused_args](const std::vector<std::uintptr_t> &mla_ptrs, const std::vector<std::uintptr_t> &idx_ptrs,
+                       std::uintptr_t workspace, size_t workspace_bytes, int64_t t, int64_t h, int64_t q_lora_rank,
+                       int64_t mla_heads, int64_t mla_cache_rows, double epsilon_cq, double epsilon_ckv, bool absorb_exact,
+                       int64_t idx_heads, int64_t idx_cache_rows, double idx_eps, std::uintptr_t stream) {
+              PtoMlaIndexerPrologQuantArgs a = fused_args(mla_ptrs, idx_ptrs, workspace, workspace_bytes, t, h, q_lora_rank,
+                                                          mla_heads, mla_cache_rows, epsilon_cq, epsilon_ckv, absorb_exact,
+                                                          idx_heads, idx_cache_rows, idx_eps);
+              check(pto_mla_indexer_prolog_quant_launch(&a, ptr<void>(stream)));
           });
 }

@@ -95,7 +95,7 @@ def _need(t: torch.Tensor, name: str, dtype, numel: Optional[int] = None):
 def lightning_indexer_prolog_quant(x_in, q_norm_in, q_norm_scale_in, w_qb_in, w_qb_scale_in, wk_in, w_proj_in,
                                    ln_gamma_k_in, ln_beta_k_in, cos_idx_rope_in, sin_idx_rope_in, hadamard_q_in,
                                    hadamard_k_in, k_int8_in, k_scale_in, k_cache_index_in, q_int8_out, q_scale_out,
-                                   k_int8_out, k_scale_out, weights_out, attrs=None, configs=None):
+                                   k_int8_out, k_scale_out, weights_out, attrs=None, configs=None, _collect=None):
     C = _native.load()
     attrs = attrs if attrs is not None else IndexerPrologQuantAttr()
     if getattr(attrs, "layerout_query", "TND") != "TND" or getattr(attrs, "layerout_key", "PA_BSND") != "PA_BSND":
@@ -154,6 +154,12 @@ def lightning_indexer_prolog_quant(x_in, q_norm_in, q_norm_scale_in, w_qb_in, w_
     copy_unless_same(kc, kc_in, "k_int8")
     copy_unless_same(ks, ks_in, "k_scale")
 
+    if _collect is not None:
+        # half of the fused operator: checked here, launched by the caller together with the other half
+        _collect.append(dict(ptrs=[v.data_ptr() for v in (x, qn, qns, wqb, wqbs, wk, wp, gam, bet, cos, sin, hq, hk, kc, ks, kidx,
+                                                          qo, qso, wo)],
+                             t=t, h=h, q_lora=q_lora, n_heads=n_heads, cache_rows=cache_rows, eps=float(attrs.eps)))
+        return None
     ws_bytes = C.li_prolog_quant_workspace_bytes(t, h, q_lora, n_heads, cache_rows)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream

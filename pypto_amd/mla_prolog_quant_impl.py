@@ -90,7 +90,7 @@ def _need(t: torch.Tensor, name: str, dtype, numel: Optional[int] = None):
 def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gamma_cq, gamma_ckv, cos, sin, cache_index,
                       kv_cache, kr_cache, k_scale_cache, q_norm_out, q_norm_scale_out, query_nope_out, query_rope_out,
                       kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv, cache_mode, tile_config,
-                      rope_cfg):
+                      rope_cfg, _collect=None):
     C = _native.load()
     if cache_mode != "PA_BSND":
         raise ValueError(f"mla_prolog_quant: cache_mode {cache_mode!r} is not built (only 'PA_BSND')")
@@ -147,6 +147,13 @@ def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gam
             raise ValueError(f"{nm} and {nm}_out differ in shape or type")
         copy_unless_same(a, b_, nm)
 
+    if _collect is not None:
+        # half of the fused operator: checked here, launched by the caller together with the other half
+        _collect.append(dict(ptrs=[v.data_ptr() for v in (x, wdq, wuq, dqs, wuk, wdkv, gcq, gckv, cs, sn, cidx, kvc, krc, ksc, qn,
+                                                          qns, qnope, qrope)],
+                             t=t, h=h, q_lora=q_lora, n_heads=n_heads, cache_rows=cache_rows, eps_cq=float(epsilon_cq),
+                             eps_ckv=float(epsilon_ckv), absorb_exact=bool(EXACT_ABSORB), device=dev))
+        return None
     ws_bytes = C.mla_prolog_quant_workspace_bytes(t, h, q_lora, n_heads, cache_rows)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
@@ -163,20 +170,20 @@ def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gam
 def mla_prolog_quant_d(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gamma_cq, gamma_ckv, cos, sin, cache_index,
                        kv_cache, kr_cache, k_scale_cache, q_norm_out, q_norm_scale_out, query_nope_out, query_rope_out,
                        kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv, cache_mode="PA_BSND",
-                       tile_config=None, rope_cfg=None):
+                       tile_config=None, rope_cfg=None, _collect=None):
     """Decode entry point (reference :798-869)."""
     return _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gamma_cq, gamma_ckv, cos, sin,
                              cache_index, kv_cache, kr_cache, k_scale_cache, q_norm_out, q_norm_scale_out, query_nope_out,
                              query_rope_out, kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv,
-                             cache_mode, tile_config, rope_cfg)
+                             cache_mode, tile_config, rope_cfg, _collect)
 
 
 def mla_prolog_quant_p(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gamma_cq, gamma_ckv, cos, sin, cache_index,
                        kv_cache, kr_cache, k_scale_cache, q_norm_out, q_norm_scale_out, query_nope_out, query_rope_out,
                        kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv, cache_mode="PA_BSND",
-                       tile_config=None, rope_cfg=None):
+                       tile_config=None, rope_cfg=None, _collect=None):
     """Prefill entry point (reference :717-788); the same kernels."""
     return _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gamma_cq, gamma_ckv, cos, sin,
                              cache_index, kv_cache, kr_cache, k_scale_cache, q_norm_out, q_norm_scale_out, query_nope_out,
                              query_rope_out, kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv,
-                             cache_mode, tile_config, rope_cfg)
+                             cache_mode, tile_config, rope_cfg, _collect)

@@ -183,3 +183,97 @@ def test_fused_mla_indexer_prolog_matches_the_oracle_chain():
     assert np.array_equal(weights.cpu().numpy().view(np.uint16), r_lip["weights"].view(np.uint16))
     assert np.array_equal(dl.k_cache.cpu().numpy(), r_lip["k_cache"])
     assert np.array_equal(dl.k_cache_scale.cpu().numpy().view(np.uint16), r_lip["k_cache_scale"].view(np.uint16))
+
+
+def test_fused_entry_point_through_the_c_abi_keeps_the_intermediates_in_its_workspace():
+    """pto_mla_indexer_prolog_quant_launch called with ctypes, q_norm_out / q_norm_scale_out NULL: the query latent
+    lives in the common workspace, and every output equals what the two operators give when called one after
+    the other (bit for bit)."""
+    import ctypes
+    import os
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs
+    lib = ctypes.CDLL(os.path.join(os.path.dirname(os.path.abspath(pypto_amd.__file__)), "libpypto_amd_sfa.so"))
+    vp, i64, f32, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int32
+
+    class Mla(ctypes.Structure):
+        _fields_ = [(n, vp) for n in ("token_x", "w_dq", "w_uq_qr", "dequant_scale", "w_uk", "w_dkv_kr", "gamma_cq", "gamma_ckv",
+                                      "cos", "sin", "cache_index", "kv_cache", "kr_cache", "k_scale_cache", "q_norm_out",
+                                      "q_norm_scale_out", "query_nope_out", "query_rope_out", "workspace")] + \
+                   [("workspace_bytes", ctypes.c_size_t)] + [(n, i64) for n in ("t", "h", "q_lora_rank", "n_heads", "cache_rows")] + \
+                   [("epsilon_cq", f32), ("epsilon_ckv", f32), ("absorb_exact", i32), ("reserved", i32)]
+
+    class Idx(ctypes.Structure):
+        _fields_ = [(n, vp) for n in ("x", "q_norm", "q_norm_scale", "w_qb", "w_qb_scale", "wk", "w_proj", "ln_gamma_k", "ln_beta_k",
+                                      "cos_idx_rope", "sin_idx_rope", "hadamard_q", "hadamard_k", "k_cache", "k_cache_scale",
+                                      "k_cache_index", "q_int8", "q_scale", "weights", "workspace")] + \
+                   [("workspace_bytes", ctypes.c_size_t)] + [(n, i64) for n in ("t", "h", "q_lora_rank", "n_heads", "cache_rows")] + \
+                   [("eps", f32), ("reserved", i32)]
+
+    class Fused(ctypes.Structure):
+        _fields_ = [("mla", Mla), ("indexer", Idx), ("workspace", vp), ("workspace_bytes", ctypes.c_size_t)]
+
+    kw = dict(h=512, q_lora_rank=512)
+    mla = gen_mla_prolog_inputs(3, 2, [300, 129, 64], seed=31, n_heads=8, **kw)
+    lip = gen_indexer_prolog_inputs(3, 2, [300, 129, 64], seed=32, n_heads=8, **kw)
+    dev = torch.device("cuda:0")
+    t, n = 6, 8
+
+    def outputs():
+        dm, dl = mla.to(dev), lip.to(dev)
+        return dm, dl, dict(q_nope=torch.zeros([t, n, 512], dtype=torch.bfloat16, device=dev),
+                            q_rope=torch.zeros([t, n, 64], dtype=torch.bfloat16, device=dev),
+                            q_int8=torch.zeros([t, n, 128], dtype=torch.int8, device=dev),
+                            q_scale=torch.zeros([t, n, 1], dtype=torch.float16, device=dev),
+                            weights=torch.zeros([t, n], dtype=torch.float16, device=dev))
+
+    # the two operators one after the other
+    dm, dl, o = outputs()
+    q_norm = torch.zeros([t, 512], dtype=torch.int8, device=dev)
+    q_norm_scale = torch.zeros([t, 1], dtype=torch.float32, device=dev)
+    pypto_amd.mla_prolog_quant_d(dm.token_x, dm.w_dq, dm.w_uq_qr, dm.dequant_scale, dm.w_uk, dm.w_dkv_kr, dm.gamma_cq, dm.gamma_ckv,
+                                 dm.cos, dm.sin, dm.cache_index, dm.kv_cache, dm.kr_cache, dm.k_scale_cache, q_norm, q_norm_scale,
+                                 o["q_nope"], o["q_rope"], dm.kv_cache, dm.kr_cache, dm.k_scale_cache, 1e-5, 1e-5)
+    pypto_amd.lightning_indexer_prolog_quant(dm.token_x, q_norm, q_norm_scale, dl.w_qb, dl.w_qb_scale, dl.wk, dl.w_proj, dl.ln_gamma_k,
+                                             dl.ln_beta_k, dm.cos, dm.sin, dl.hadamard_q, dl.hadamard_k, dl.k_cache, dl.k_cache_scale,
+                                             dm.cache_index, o["q_int8"], o["q_scale"], dl.k_cache, dl.k_cache_scale, o["weights"])
+    torch.cuda.synchronize()
+    want = {k: v.clone() for k, v in o.items()}
+    want.update(kv=dm.kv_cache.clone(), kr=dm.kr_cache.clone(), ks=dm.k_scale_cache.clone(), kc=dl.k_cache.clone(), kcs=dl.k_cache_scale.clone())
+
+    # the fused entry point
+    dm, dl, o = outputs()
+    a = Fused()
+    for name, ten in (("token_x", dm.token_x), ("w_dq", dm.w_dq), ("w_uq_qr", dm.w_uq_qr), ("dequant_scale", dm.dequant_scale),
+                      ("w_uk", dm.w_uk), ("w_dkv_kr", dm.w_dkv_kr), ("gamma_cq", dm.gamma_cq), ("gamma_ckv", dm.gamma_ckv),
+                      ("cos", dm.cos), ("sin", dm.sin), ("cache_index", dm.cache_index), ("kv_cache", dm.kv_cache),
+                      ("kr_cache", dm.kr_cache), ("k_scale_cache", dm.k_scale_cache), ("query_nope_out", o["q_nope"]),
+                      ("query_rope_out", o["q_rope"])):
+        setattr(a.mla, name, ten.data_ptr())
+    a.mla.t, a.mla.h, a.mla.q_lora_rank, a.mla.n_heads = t, 512, 512, n
+    a.mla.cache_rows = dm.kv_cache.shape[0] * dm.kv_cache.shape[1]
+    a.mla.epsilon_cq = a.mla.epsilon_ckv = 1e-5
+    a.mla.absorb_exact = 1                                   # the autouse fixture runs the separate operators that way
+    for name, ten in (("w_qb", dl.w_qb), ("w_qb_scale", dl.w_qb_scale), ("wk", dl.wk), ("w_proj", dl.w_proj),
+                      ("ln_gamma_k", dl.ln_gamma_k), ("ln_beta_k", dl.ln_beta_k), ("hadamard_q", dl.hadamard_q),
+                      ("hadamard_k", dl.hadamard_k), ("k_cache", dl.k_cache), ("k_cache_scale", dl.k_cache_scale),
+                      ("q_int8", o["q_int8"]), ("q_scale", o["q_scale"]), ("weights", o["weights"])):
+        setattr(a.indexer, name, ten.data_ptr())
+    a.indexer.n_heads = n
+    a.indexer.cache_rows = dl.k_cache.shape[0] * dl.k_cache.shape[1]
+    a.indexer.eps = 1e-6
+    need = ctypes.c_size_t()
+    assert lib.pto_mla_indexer_prolog_quant_workspace_bytes(ctypes.byref(a), ctypes.byref(need)) == 0
+    ws = torch.empty(need.value, dtype=torch.uint8, device=dev)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), need.value
+    lib.pto_last_error.restype = ctypes.c_char_p
+    rc = lib.pto_mla_indexer_prolog_quant_launch(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0, lib.pto_last_error()
+    torch.cuda.synchronize()
+    got = dict(o, kv=dm.kv_cache, kr=dm.kr_cache, ks=dm.k_scale_cache, kc=dl.k_cache, kcs=dl.k_cache_scale)
+    for k in want:
+        assert torch.equal(got[k].view(torch.uint8), want[k].view(torch.uint8)), k
+    # the intermediates sit at the front of the workspace
+    assert torch.equal(ws[:t * 512].view(torch.int8).view(t, 512), q_norm)
+    # a workspace one byte short is refused, nothing is launched
+    a.workspace_bytes = need.value - 1
+    assert lib.pto_mla_indexer_prolog_quant_launch(ctypes.byref(a), None) == -2
