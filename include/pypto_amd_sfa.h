@@ -396,8 +396,9 @@ int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *args, void *hip_str
  *            cos_idx_rope, sin_idx_rope, k_cache_index, t, h, q_lora_rank, workspace and
  *            workspace_bytes are ignored: taken from the MLA part and the common workspace.
  *   workspace  pto_mla_indexer_prolog_quant_workspace_bytes() bytes, 256-byte aligned: the
- *            intermediates and one area that serves the partial sums of both halves in turn.
- * Six kernels on the given stream, nothing else; errors as for the two operators.
+ *            intermediates, then the partial sums of the MLA half, then those of the indexer half.
+ * Five kernels on the given stream, nothing else (the last launches of the two halves do not
+ * depend on each other and run as one); errors as for the two operators.
  */
 typedef struct PtoMlaIndexerPrologQuantArgs {
     PtoMlaPrologQuantArgs mla;

@@ -15,7 +15,7 @@ LIB_NAME = "libpypto_amd_sfa.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 EXT_PATH = os.path.join(HERE, "_C" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
 
-HIP_SOURCES = ["sfa_kernels.hip", "li_kernels.hip", "lip_kernels.hip", "mlap_kernels.hip", "capi.cpp"]
+HIP_SOURCES = ["sfa_kernels.hip", "li_kernels.hip", "lip_kernels.hip", "mlap_kernels.hip", "prolog_fused.hip", "capi.cpp"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # fuse a*b+c only where the source writes it in one expression; files that need exact

@@ -13,6 +13,7 @@
 
 #include "li_kernels.h"
 #include "lip_kernels.h"
+#include "prolog_fused.h"
 #include "mlap_kernels.h"
 #include "sfa_kernels.h"
 
@@ -508,7 +509,8 @@ int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *a, size_t *b
     return PTO_OK;
 }
 
-int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
+// checked arguments -> kernel parameters
+static int lip_params(const PtoLiPrologQuantArgs *a, pto::LipParams &p)
 {
     int rc = lip_check(a);
     if (rc != PTO_OK) return rc;
@@ -526,7 +528,6 @@ int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
         if (reinterpret_cast<uintptr_t>(ptr) & 15)
             return fail(PTO_E_INVALID_ARG, "li_prolog: tensor and workspace pointers must be 16-byte aligned");
 
-    pto::LipParams p;
     p.x = static_cast<const uint16_t *>(a->x);
     p.q_norm = a->q_norm;
     p.q_norm_scale = a->q_norm_scale;
@@ -556,6 +557,14 @@ int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
     p.eps = a->eps;
     p.w_mul0 = (float)std::pow((double)a->n_heads, -0.5);
     p.w_mul1 = (float)std::pow((double)pto::LIP_DIM, -0.5);
+    return PTO_OK;
+}
+
+int pto_li_prolog_quant_launch(const PtoLiPrologQuantArgs *a, void *hip_stream)
+{
+    pto::LipParams p;
+    int rc = lip_params(a, p);
+    if (rc != PTO_OK) return rc;
     hipError_t e = pto::lip_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "li_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
@@ -570,7 +579,8 @@ int pto_mla_prolog_quant_workspace_bytes(const PtoMlaPrologQuantArgs *a, size_t 
     return PTO_OK;
 }
 
-int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream)
+// checked arguments -> kernel parameters
+static int mlap_params(const PtoMlaPrologQuantArgs *a, pto::MlapParams &p)
 {
     int rc = mlap_check(a);
     if (rc != PTO_OK) return rc;
@@ -589,7 +599,6 @@ int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream
         if (reinterpret_cast<uintptr_t>(ptr) & 15)
             return fail(PTO_E_INVALID_ARG, "mla_prolog: tensor and workspace pointers must be 16-byte aligned");
 
-    pto::MlapParams p;
     p.x = static_cast<const uint16_t *>(a->token_x);
     p.w_dq = static_cast<const uint16_t *>(a->w_dq);
     p.w_uqqr = a->w_uq_qr;
@@ -618,6 +627,14 @@ int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream
     p.eps_cq = a->epsilon_cq;
     p.eps_ckv = a->epsilon_ckv;
     p.absorb_exact = a->absorb_exact ? 1 : 0;
+    return PTO_OK;
+}
+
+int pto_mla_prolog_quant_launch(const PtoMlaPrologQuantArgs *a, void *hip_stream)
+{
+    pto::MlapParams p;
+    int rc = mlap_params(a, p);
+    if (rc != PTO_OK) return rc;
     hipError_t e = pto::mlap_launch(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
@@ -656,8 +673,9 @@ int fused_plan(const PtoMlaIndexerPrologQuantArgs *a, FusedPlan *pl)
     pl->q_norm_off = 0;
     pl->q_norm_scale_off = qn;
     pl->rest_off = qn + qs;
-    // the MLA prolog's partial sums are dead when the indexer prolog's kernels start: one area serves both
-    pl->total = qn + qs + (w_mla > w_idx ? w_mla : w_idx);
+    // the partial sums of both halves are alive at once (the last launch finishes both), so each has its own area
+    const size_t w_mla_pad = (w_mla + 255) & ~(size_t)255;
+    pl->total = qn + qs + w_mla_pad + w_idx;
     char *base = static_cast<char *>(a->workspace);
     if (base) {
         int8_t *q_norm = a->mla.q_norm_out ? a->mla.q_norm_out : reinterpret_cast<int8_t *>(base + pl->q_norm_off);
@@ -668,7 +686,7 @@ int fused_plan(const PtoMlaIndexerPrologQuantArgs *a, FusedPlan *pl)
         pl->idx.q_norm_scale = q_norm_scale;
         pl->mla.workspace = base + pl->rest_off;
         pl->mla.workspace_bytes = w_mla;
-        pl->idx.workspace = base + pl->rest_off;
+        pl->idx.workspace = base + pl->rest_off + w_mla_pad;
         pl->idx.workspace_bytes = w_idx;
     }
     return PTO_OK;
@@ -696,9 +714,16 @@ int pto_mla_indexer_prolog_quant_launch(const PtoMlaIndexerPrologQuantArgs *a, v
                     a->workspace ? a->workspace_bytes : (size_t)0);
     if (reinterpret_cast<uintptr_t>(a->workspace) & 255)
         return fail(PTO_E_INVALID_ARG, "mla_indexer_prolog: the workspace must be 256-byte aligned");
-    rc = pto_mla_prolog_quant_launch(&pl.mla, hip_stream);
+    pto::MlapParams pm;
+    pto::LipParams pi;
+    rc = mlap_params(&pl.mla, pm);
     if (rc != PTO_OK) return rc;
-    return pto_li_prolog_quant_launch(&pl.idx, hip_stream);
+    rc = lip_params(&pl.idx, pi);
+    if (rc != PTO_OK) return rc;
+    // five launches: the last ones of the two halves do not depend on each other and run as one
+    hipError_t e = pto::prolog_fused_launch(pm, pi, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_indexer_prolog: launch failed: %s", hipGetErrorString(e));
+    return PTO_OK;
 }
 
 }  // extern "C"

@@ -46,5 +46,8 @@ struct MlapParams {
 };
 
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
+// all launches but the last, and the number of workgroups of the last (for the fused operator's last launch)
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream);
+int mlap_finish_wgs(const MlapParams &p);
 
 }  // namespace pto

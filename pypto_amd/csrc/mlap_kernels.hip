@@ -25,6 +25,7 @@
 //                        slice (staged in LDS by LDS-DMA), one output column per lane, 8 tokens at once.
 #include "mlap_kernels.h"
 #include "prolog_common.h"
+#include "prolog_finish.h"
 
 #pragma clang fp contract(off)
 
@@ -283,162 +284,18 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njo
 }
 
 // ---------------------------------------------------------------------------------------------
-constexpr int FIN_W_BYTES = MLAP_NOPE * 64 * 2;    // a wave's slice of w_uk[head]: 128 rows x 64 columns bf16
-
-// Workgroup (head, half of the 512 output columns, block of 8 tokens); wave w owns output columns
-// colbase + 64w + l.
+// Last launch: prolog_finish.h.
 __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t wsl[4 * FIN_W_BYTES];
-    __shared__ __attribute__((aligned(16))) float arow[MLAP_XTOK][MLAP_NOPE];
-    __shared__ __attribute__((aligned(16))) uint16_t abf[MLAP_XTOK][MLAP_NOPE];      // the same values as bf16 (they are bf16-valued)
-    const int l = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int head = blockIdx.x % p.n_heads;
-    const int half = (blockIdx.x / p.n_heads) & 1;
-    const int t0 = (blockIdx.x / p.n_heads / 2) * MLAP_XTOK;
-    const int ncols = p.n_heads * MLAP_QHEAD;
-    const int colbase = half * 256 + 64 * w;
-
-    {   // this wave's slice: rows of 128 bytes, pitch 1024 bytes: 8 lanes per row, 8 rows per request
-        const uint8_t *src = reinterpret_cast<const uint8_t *>(p.w_uk) + ((size_t)head * MLAP_NOPE + (l >> 3)) * (MLAP_KV * 2) +
-                             colbase * 2 + 16 * (l & 7);
-        const uint32_t dst = (uint32_t)(uintptr_t)(lds_byte_t *)(wsl + w * FIN_W_BYTES);
-#pragma unroll 1
-        for (int i = 0; i < MLAP_NOPE / 8; ++i) dma16(src + (size_t)i * 8 * MLAP_KV * 2, dst + 1024 * i);
-    }
-    // the head's query channels of tokens t0 + w and t0 + 4 + w: partial sums added, de-quantised, bf16
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-        const int tl = 4 * u + w;
-        const int t = t0 + tl;
-        const int tt = t < p.T ? t : p.T - 1;
-        const float ts = p.q_norm_scale[tt];
-        // nope part: lane l -> channels 2l, 2l+1
-        {
-            const int col = head * MLAP_QHEAD + 2 * l;
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
-                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + tt) * ncols + col);
-                s0 += v.x;
-                s1 += v.y;
-            }
-            const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
-            f32x2 av = {bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0])),
-                        bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]))};
-            *reinterpret_cast<f32x2 *>(&arow[tl][2 * l]) = av;
-            *reinterpret_cast<uint32_t *>(&abf[tl][2 * l]) = pack_bf16x2(av[0], av[1]);
-        }
-        // rope part (first half-workgroup only): lane l < 32 -> channels 2l, 2l+1 = rotation partners l, 32+l
-        if (half == 0 && l < 32 && t < p.T) {
-            const int col = head * MLAP_QHEAD + MLAP_NOPE + 2 * l;
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
-                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + t) * ncols + col);
-                s0 += v.x;
-                s1 += v.y;
-            }
-            const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
-            const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
-            const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
-            const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
-            const float sn0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), sn1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
-            const float r0 = __builtin_fmaf(v0, c0, (-v1) * sn0);
-            const float r1 = __builtin_fmaf(v1, c1, v0 * sn1);
-            uint16_t *out = p.q_rope + ((size_t)t * p.n_heads + head) * MLAP_ROPE;
-            out[l] = (uint16_t)(pack_bf16x2(r0, 0.f) & 0xffffu);
-            out[32 + l] = (uint16_t)(pack_bf16x2(r1, 0.f) & 0xffffu);
-        }
-    }
-    VM_WAIT(0);
-    __syncthreads();
-
-    if (!p.absorb_exact) {
-        // On the matrix cores: C^T[col][token] = sum_i W^T[col][i] a^T[i][token], v_mfma_f32_32x32x16_bf16 with
-        // A = the wave's slice of w_uk read transposed out of LDS (ds_read_b64_tr_b16: lane (col, half) gets rows
-        // 16ks + 4*half + 0..3 and 16ks + 8 + 4*half + 0..3 of its column), B = the tokens' query values in the same
-        // row order (lanes of tokens 8..31 repeat token 0; their results are not stored).  Two blocks of 32
-        // columns, eight contraction steps.  Lane (token, half) then holds columns 8*(r/4) + 4*half + r%4 of a block.
-        const uint16_t *wt = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) +
-                             (4 * (l >> 5) + ((l & 15) >> 2)) * 64 + 16 * ((l >> 4) & 1) + 4 * (l & 3);
-        const int tok = (l & 31) < MLAP_XTOK ? (l & 31) : 0;
-        const uint16_t *at = &abf[tok][4 * (l >> 5)];
-        f32x16 c[2];
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) c[cb][r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < MLAP_NOPE / 16; ++ks) {
-            const u32x2 b0 = *reinterpret_cast<const u32x2 *>(at + 16 * ks);
-            const u32x2 b1 = *reinterpret_cast<const u32x2 *>(at + 16 * ks + 8);
-            const u32x4 bq = {b0[0], b0[1], b1[0], b1[1]};
-#pragma unroll
-            for (int cb = 0; cb < 2; ++cb) {
-                const s16x4 a0 = lds_read_tr16(wt + (16 * ks) * 64 + 32 * cb);
-                const s16x4 a1 = lds_read_tr16(wt + (16 * ks + 8) * 64 + 32 * cb);
-                const s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
-                c[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, bq), c[cb], 0, 0, 0);
-            }
-        }
-        const int t = t0 + (l & 31);
-        if ((l & 31) < MLAP_XTOK && t < p.T) {
-            uint16_t *dst = p.q_nope + ((size_t)t * p.n_heads + head) * MLAP_KV + colbase + 4 * (l >> 5);
-#pragma unroll
-            for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const u32x2 v = {pack_bf16x2(c[cb][4 * q], c[cb][4 * q + 1]), pack_bf16x2(c[cb][4 * q + 2], c[cb][4 * q + 3])};
-                    *reinterpret_cast<u32x2 *>(dst + 32 * cb + 8 * q) = v;
-                }
-        }
-        return;
-    }
-    // out[t][colbase + 64w + l] = sum_i a[t][i] * w_uk[head][i][col], i ascending; 8 tokens at once.
-    // Chunks of four rows are read one chunk ahead of the multiply-adds that consume them.
-    const uint16_t *wl = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) + l;
-    float acc[MLAP_XTOK];
-#pragma unroll
-    for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = 0.f;
-    struct Chunk {
-        f32x4 a[MLAP_XTOK];
-        uint16_t w[4];
-    };
-    auto load = [&](Chunk &c, const int i) {
-#pragma unroll
-        for (int t = 0; t < MLAP_XTOK; ++t) c.a[t] = *reinterpret_cast<const f32x4 *>(&arow[t][i]);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) c.w[j] = wl[(i + j) * 64];
-    };
-    auto fma = [&](const Chunk &c) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float wv = bf16_bits_to_f32(c.w[j]);
-#pragma unroll
-            for (int t = 0; t < MLAP_XTOK; ++t) acc[t] = __builtin_fmaf(c.a[t][j], wv, acc[t]);
-        }
-    };
-    Chunk c0, c1;
-    load(c0, 0);
-#pragma unroll 1
-    for (int i = 0; i < MLAP_NOPE; i += 8) {
-        load(c1, i + 4);
-        fma(c0);
-        load(c0, i + 8 < MLAP_NOPE ? i + 8 : 0);
-        fma(c1);
-    }
-#pragma unroll
-    for (int t = 0; t < MLAP_XTOK; ++t)
-        if (t0 + t < p.T)
-            p.q_nope[((size_t)(t0 + t) * p.n_heads + head) * MLAP_KV + colbase + l] = (uint16_t)(pack_bf16x2(acc[t], 0.f) & 0xffffu);
+    __shared__ __attribute__((aligned(16))) uint8_t lds[MLAP_FIN_LDS];
+    mlap_finish_body(p, (int)blockIdx.x, lds);
 }
-
 
 }  // namespace
 
-hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
+int mlap_finish_wgs(const MlapParams &p) { return p.n_heads * 2 * ((p.T + MLAP_XTOK - 1) / MLAP_XTOK); }
+
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
 {
     const int nblk = p.h / MLAP_XBLOCK;
     const int ngroups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
@@ -466,9 +323,14 @@ hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
     case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
     default: return hipErrorInvalidValue;
     }
-    e = hipGetLastError();
+    return hipGetLastError();
+}
+
+hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
+{
+    hipError_t e = mlap_launch_front(p, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)(p.n_heads * 2 * tgroups)), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)mlap_finish_wgs(p)), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

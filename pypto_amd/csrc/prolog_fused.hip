@@ -1,0 +1,47 @@
+// MLA prolog + lightning-indexer prolog as one operator (mla_indexer_prolog_quant_d/_p of the reference,
+// examples/models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:141-256): the kernels of the two prologs in
+// the order hidden-axis sums -> norms and quantisation of the latents -> int8 projection of the attention query ->
+// first launch of the indexer prolog, and then ONE last launch for both: the workgroups that finish the attention
+// query (absorb product, 70 KB of LDS, four waves) and those that finish the indexer's query rows, key row and
+// weights (54 KB, eight waves) do not depend on each other and fit a compute unit together, so they run side by
+// side instead of one launch after the other.
+#include "prolog_finish.h"
+
+#include "prolog_fused.h"
+
+namespace pto {
+namespace {
+
+constexpr int FUSED_FIN_LDS = MLAP_FIN_LDS > LIP_FIN_LDS ? MLAP_FIN_LDS : LIP_FIN_LDS;
+static_assert(2 * FUSED_FIN_LDS <= 160 * 1024, "two workgroups of the last launch share a compute unit");
+
+// Workgroups [0, mla_wgs): the MLA prolog's last launch (its 256 threads; the other four waves leave at once,
+// the barriers of a workgroup count the waves that are still alive).  The rest: the indexer prolog's second launch.
+__global__ __launch_bounds__(64 * FIN_WAVES) void prolog_fused_finish_kernel(const MlapParams pm, const LipParams pl, const int mla_wgs,
+                                                                             const int q_wgs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FUSED_FIN_LDS];
+    if ((int)blockIdx.x < mla_wgs) {
+        if (threadIdx.x >= 256) return;
+        mlap_finish_body(pm, (int)blockIdx.x, lds);
+    } else {
+        lip_finish_body(pl, q_wgs, (int)blockIdx.x - mla_wgs, lds);
+    }
+}
+
+}  // namespace
+
+hipError_t prolog_fused_launch(const MlapParams &pm, const LipParams &pl, hipStream_t stream)
+{
+    hipError_t e = mlap_launch_front(pm, stream);
+    if (e != hipSuccess) return e;
+    e = lip_launch_linear(pl, stream);
+    if (e != hipSuccess) return e;
+    const int mla_wgs = mlap_finish_wgs(pm);
+    const int q_wgs = lip_finish_query_wgs(pl);
+    hipLaunchKernelGGL(prolog_fused_finish_kernel, dim3((unsigned)(mla_wgs + q_wgs + pl.T)), dim3(64 * FIN_WAVES), 0, stream, pm, pl,
+                       mla_wgs, q_wgs);
+    return hipGetLastError();
+}
+
+}  // namespace pto

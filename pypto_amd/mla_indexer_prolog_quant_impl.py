@@ -4,8 +4,9 @@ Same callables, argument names and order as ``mla_indexer_prolog_quant_d`` / ``m
 the reference example (examples/models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:49-138, 141-256): the
 MLA prolog runs first; its int8 normalised query latent and that latent's scale -- intermediates the caller
 never sees (:218-219) -- are the indexer prolog's ``q_norm`` / ``q_norm_scale``; hidden states, rope tables and
-cache index are shared.  One launch call of the library (``pto_mla_indexer_prolog_quant_launch``: six kernels back to
-back on the current stream) and one workspace, in which the two intermediates live; see the two operators'
+cache index are shared.  One launch call of the library (``pto_mla_indexer_prolog_quant_launch``: five kernels on the
+current stream, the last launches of the two halves merged into one) and one workspace, in which the two
+intermediates live; see the two operators'
 modules for layouts and for what is built.  Returns ``None``.
 """
 from __future__ import annotations
@@ -38,7 +39,7 @@ def _fused(mla_op, token_x, mla_w_dq, mla_w_uq_qr, mla_dequant_scale, mla_w_uk, 
     t, h = x.shape
     q_lora_rank = w_qb.shape[0]
     # one workspace for the whole operator: the int8 query latent and its scale (the intermediates the caller
-    # never sees) in front, then one area that serves the partial sums of both halves in turn
+    # never sees) in front, then the partial sums of the two halves
     ws_bytes = C.mla_indexer_prolog_quant_workspace_bytes(t, h, q_lora_rank, w_uk.shape[0], kvc.shape[0] * kvc.shape[1],
                                                           w_proj.shape[1], kc.shape[0] * kc.shape[1])
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
