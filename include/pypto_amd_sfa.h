@@ -132,7 +132,7 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
  * the process ends) instead of a workspace; args->workspace and workspace_bytes
  * are ignored.  Nothing is allocated or freed; the first call on a device looks
  * the array's device address up.  A shape whose splits need more than the array
- * holds is refused with PTO_E_WORKSPACE (every BASELINE decode shape fits: 32
+ * holds is refused with PTO_E_WORKSPACE (the decode shapes this library is benchmarked on fit: 32
  * rows x 8 splits and 128 rows x 2 splits of 128 heads take 33.8 MB).
  * All calls on one GPU share the array: calls whose execution may overlap (two
  * streams, two threads) race on it and must use pto_sfa_quant_launch with
