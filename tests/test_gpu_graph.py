@@ -113,3 +113,70 @@ def test_prologs_replays_match_eager():
         want = list(o_e) + caches
         for i, (g_, w_) in enumerate(zip(got, want)):
             assert torch.equal(g_.view(torch.uint8), w_.view(torch.uint8)), f"replay {rep}: output {i} differs from the eager call"
+
+
+def test_fused_prolog_operator_replays_match_the_two_operators_called_eagerly():
+    """mla_indexer_prolog_quant_d (one library call, one workspace from torch's pool, the last launches of the two
+    halves merged) recorded once and replayed with new hidden states: every replay equals the two separate
+    operators called eagerly on the same inputs, bit for bit."""
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
+    dev = torch.device(DEV)
+    b, s1, act = 4, 2, [5000, 300, 129, 64]
+    kw = dict(h=512, q_lora_rank=1536)
+    mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=8, **kw).to(dev)
+    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=4, **kw).to(dev)
+    t = b * s1
+    caches = [mla.kv_cache, mla.kr_cache, mla.k_scale_cache, lip.k_cache, lip.k_cache_scale]
+    base = [c.clone() for c in caches]
+
+    def outputs():
+        return (torch.zeros(t, 8, 512, dtype=torch.bfloat16, device=dev), torch.zeros(t, 8, 64, dtype=torch.bfloat16, device=dev),
+                torch.zeros(t, 4, 128, dtype=torch.int8, device=dev), torch.zeros(t, 4, 1, dtype=torch.float16, device=dev),
+                torch.zeros(t, 4, dtype=torch.float16, device=dev))
+
+    def fused(o):
+        qnope, qrope, iq, iqs, iw = o
+        pypto_amd.mla_indexer_prolog_quant_d(
+            mla.token_x, mla.w_dq, mla.w_uq_qr, mla.dequant_scale, mla.w_uk, mla.w_dkv_kr, mla.gamma_cq, mla.gamma_ckv, mla.cos,
+            mla.sin, mla.cache_index, mla.kv_cache, mla.kr_cache, mla.k_scale_cache, lip.w_qb, lip.w_qb_scale, lip.wk, lip.w_proj,
+            lip.ln_gamma_k, lip.ln_beta_k, lip.hadamard_q, lip.hadamard_k, lip.k_cache, lip.k_cache_scale, qnope, qrope,
+            mla.kv_cache, mla.kr_cache, mla.k_scale_cache, iq, iqs, lip.k_cache, lip.k_cache_scale, iw, 1e-5, 1e-5, "PA_BSND",
+            None, None, None, None)
+
+    def separate(o):
+        qnope, qrope, iq, iqs, iw = o
+        qn = torch.zeros(t, 1536, dtype=torch.int8, device=dev)
+        qs = torch.zeros(t, 1, device=dev)
+        pypto_amd.mla_prolog_quant_d(mla.token_x, mla.w_dq, mla.w_uq_qr, mla.dequant_scale, mla.w_uk, mla.w_dkv_kr, mla.gamma_cq,
+                                     mla.gamma_ckv, mla.cos, mla.sin, mla.cache_index, mla.kv_cache, mla.kr_cache,
+                                     mla.k_scale_cache, qn, qs, qnope, qrope, mla.kv_cache, mla.kr_cache, mla.k_scale_cache,
+                                     1e-5, 1e-5, "PA_BSND", None, None)
+        pypto_amd.lightning_indexer_prolog_quant(mla.token_x, qn, qs, lip.w_qb, lip.w_qb_scale, lip.wk, lip.w_proj, lip.ln_gamma_k,
+                                                 lip.ln_beta_k, mla.cos, mla.sin, lip.hadamard_q, lip.hadamard_k, lip.k_cache,
+                                                 lip.k_cache_scale, mla.cache_index, iq, iqs, lip.k_cache, lip.k_cache_scale, iw)
+
+    o_g, o_e = outputs(), outputs()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fused(o_g)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fused(o_g)
+    gen = torch.Generator().manual_seed(19)
+    for rep in range(3):
+        mla.token_x.copy_(torch.randn(mla.token_x.shape, generator=gen).to(torch.bfloat16))
+        for c, b0 in zip(caches, base):
+            c.copy_(b0)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in o_g] + [c.clone() for c in caches]
+        for c, b0 in zip(caches, base):
+            c.copy_(b0)
+        separate(o_e)
+        torch.cuda.synchronize()
+        want = list(o_e) + caches
+        for i, (g_, w_) in enumerate(zip(got, want)):
+            assert torch.equal(g_.view(torch.uint8), w_.view(torch.uint8)), f"replay {rep}: output {i} differs from the separate operators"
