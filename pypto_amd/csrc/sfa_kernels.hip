@@ -36,6 +36,16 @@ constexpr int PITCH = D + 8;      // LDS row pitch in bf16 elements (1168 B: row
 constexpr int KSTEPS = D / 16;    // 36 contraction steps of 16
 constexpr int DVB = DN / 32;      // 16 output blocks of 32 value channels
 
+// Row i of a tile's score operand (and of the score accumulator) is key tile_row_of(i) of the tile: the two
+// middle bits of i move below its two lowest.  A transposing V^T read then addresses keys r, r+4, r+8, r+12
+// with each of its half-waves, four rows whose 64-byte pieces lie 16 banks apart at this pitch, instead of
+// four neighbouring rows whose pieces overlap pairwise; any 16 consecutive keys, in whatever order, still
+// serve the 16-byte score operand reads without a conflict.
+__device__ __forceinline__ constexpr int tile_row_of(const int i)
+{
+    return (i & 16) | ((i & 3) << 2) | ((i >> 2) & 3);
+}
+
 // Four int8 (one dword) times one scale -> four bf16 in two registers.
 // x*sc is formed as fma(float(x + 128), sc, -128*sc): the byte is biased to unsigned so that a single
 // v_cvt_f32_ubyteN converts it, and the fused multiply-add rounds the exact product (x*sc) once, which
@@ -545,7 +555,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
         {
-            const uint16_t *arow = cur_tile + col * PITCH + 8 * half;
+            const uint16_t *arow = cur_tile + tile_row_of(col) * PITCH + 8 * half;
             bf16x8 fa[2][4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) fa[0][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * e);
@@ -573,7 +583,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         if (kt + KT > k_end) {                  // only the split's last tile can hold keys past k_end
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if (kt + 8 * (r >> 2) + 4 * half + (r & 3) >= k_end) s[r] = -INFINITY;
+                if (kt + tile_row_of(8 * (r >> 2) + 4 * half + (r & 3)) >= k_end) s[r] = -INFINITY;
         }
         // the scale is positive here (its sign went into Q^T), so the largest raw score gives the largest
         // scaled one and the scaling itself is folded into the exponent's multiply-add
@@ -630,12 +640,12 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead;
         // interleaved with the de-quantisation of the next tile into the other buffer
         {
-            const uint16_t *vbase = cur_tile + (4 * half + ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+            const uint16_t *vbase = cur_tile + (half + 4 * ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
             s16x4 va[2][4][2];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 va[0][e][0] = lds_read_tr16(vbase + 32 * e);
-                va[0][e][1] = lds_read_tr16(vbase + 32 * e + 8 * PITCH);
+                va[0][e][1] = lds_read_tr16(vbase + 32 * e + 2 * PITCH);
             }
 #pragma unroll
             for (int g = 0; g < 8; ++g) {
@@ -646,7 +656,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
                         const int m = 4 * (g + 1) + e;
                         const uint16_t *a0 = vbase + (16 * (m >> 4)) * PITCH + 32 * (m & 15);
                         va[(g + 1) & 1][e][0] = lds_read_tr16(a0);
-                        va[(g + 1) & 1][e][1] = lds_read_tr16(a0 + 8 * PITCH);
+                        va[(g + 1) & 1][e][1] = lds_read_tr16(a0 + 2 * PITCH);
                     }
                 }
 #pragma unroll
