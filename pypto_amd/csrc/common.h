@@ -65,6 +65,17 @@ __device__ __forceinline__ void dma16(const void *gaddr, const uint32_t lds_dst)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gaddr), "s"(dst) : "memory", "m0");
 }
 
+// the same for the lanes of a mask only (the others request and write nothing); the mask is applied
+// inside the statement, so no branch splits the caller's instruction stream
+__device__ __forceinline__ void dma16_lanes(const void *gaddr, const uint32_t lds_dst, const uint64_t lanes)
+{
+    const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %3\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, off\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved) : "v"(gaddr), "s"(dst), "s"(lanes) : "memory", "m0");
+}
+
 // four bytes per lane: lane i's dword at gaddr lands at lds_dst + 4*i
 __device__ __forceinline__ void dma4(const void *gaddr, const uint32_t lds_dst)
 {

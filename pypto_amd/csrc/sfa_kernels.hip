@@ -167,13 +167,17 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     const int b = t / p.S1;
     const int s1i = t - b * p.S1;
 
-    int cur = p.act[b] - p.S1 + 1 + s1i;
-    cur = cur < 0 ? 0 : (cur > p.topk ? p.topk : cur);
-    const int ntile = (cur + KT - 1) / KT;
-    const int tiles_per_split = (ntile + p.nsplit - 1) / p.nsplit;
-    const int k_begin = sp * tiles_per_split * KT;
-    int k_end = k_begin + tiles_per_split * KT;
-    k_end = k_end > cur ? cur : k_end;
+    // The sequence length is asked for here and looked at only after the first requests below are on their
+    // way: the memory latency of this load would otherwise stand in front of everything else.
+    const int act_b = p.act[b];
+    // keys [kb, ke) of a row with n selected keys that this split takes
+    auto split_keys = [&](const int n, int &kb, int &ke) {
+        const int ntile = (n + KT - 1) / KT;
+        const int tiles_per_split = (ntile + p.nsplit - 1) / p.nsplit;
+        kb = sp * tiles_per_split * KT;
+        ke = kb + tiles_per_split * KT;
+        ke = ke > n ? n : ke;
+    };
 
     const int head = hg * (32 * NW) + w * 32 + col;
     const bool head_ok = head < p.NQ;
@@ -248,11 +252,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // table) ahead of the gather itself.  When the table fits two entries per thread both loads travel
     // as LDS-DMA requests between the Q^T passes, waited for by count, so that the chain runs beside
     // the Q^T staging instead of after it; each lane handles the entries it requested itself.
-    const int n_valid = k_end - k_begin;
-    const int n_pad = n_valid > 0 ? (n_valid + 2 * KT - 1) / (2 * KT) * (2 * KT) + 2 * KT : 0;
     constexpr int FAST_ENTRIES = 2 * NW * 64;
     static_assert(2 * FAST_ENTRIES <= SFA_MAX_CHUNK + 3 * KT, "positions and pages of the short table share its memory");
-    const bool fast = n_valid > 0 && n_pad <= FAST_ENTRIES;                    // uniform
+    auto padded = [](const int n) { return n > 0 ? (n + 2 * KT - 1) / (2 * KT) * (2 * KT) + 2 * KT : 0; };
     const int wave_first = __builtin_amdgcn_readfirstlane(w) * 64;
     auto row_of = [&](const int idx, const int page) {
         long long row = (long long)page * p.bs + (idx - (idx / p.bs) * p.bs);
@@ -263,17 +265,39 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         const int blk = idx / p.bs;
         return blk < 0 ? 0 : (blk >= p.maxblk ? p.maxblk - 1 : blk);
     };
-    if (fast) {
+    auto request_positions = [&](const int kb, const int nv) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int i = tid + j * NW * 64;
-            dma4(p.topk_idx + (size_t)t * p.topk + k_begin + (i < n_valid ? i : 0),
+            dma4(p.topk_idx + (size_t)t * p.topk + kb + (i < nv ? i : 0),
                  (uint32_t)(uintptr_t)(lds_byte_t *)(rows_lds + j * NW * 64 + wave_first));
         }
-    }
+    };
+    // A decoding row nearly always sees all topk selected keys.  The positions of this split are requested on
+    // that assumption before the sequence length has arrived, which takes one memory latency out of the chain
+    // length -> positions -> pages -> rows -> first tile; if the length says otherwise they are requested
+    // again (same destinations; requests complete in order, so the later ones stand).
+    int kb_s, ke_s;
+    split_keys(p.topk, kb_s, ke_s);
+    const int nv_s = ke_s - kb_s;
+    const bool fast_s = nv_s > 0 && padded(nv_s) <= FAST_ENTRIES;              // uniform
+    if (fast_s) request_positions(kb_s, nv_s);
     request_q(0);                                                             // 16 requests
+    int cur = act_b - p.S1 + 1 + s1i;
+    cur = cur < 0 ? 0 : (cur > p.topk ? p.topk : cur);
+    int k_begin, k_end;
+    split_keys(cur, k_begin, k_end);
+    const int n_valid = k_end - k_begin;
+    const int n_pad = padded(n_valid);
+    const bool fast = n_valid > 0 && n_pad <= FAST_ENTRIES;                    // uniform
+    const bool as_assumed = fast_s && k_begin == kb_s && n_valid == nv_s;     // uniform
     if (fast) {
-        __builtin_amdgcn_s_waitcnt(vmcnt_imm(16));                            // the positions have landed
+        if (as_assumed) {
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(16));                        // the positions have landed
+        } else {
+            request_positions(k_begin, n_valid);
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+        }
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -350,7 +374,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         if (k < KPW / 2) {
             dma16(p.kn + (size_t)row * p.kn_pitch + 16 * col, dst + (wu * KPW + 2 * k) * DN);
         } else if (k == KPW / 2) {
-            if (l < KPW) dma16(p.ksc + (size_t)row * p.ksc_pitch, dst + STG_NOPE + wu * KPW * 16);
+            dma16_lanes(p.ksc + (size_t)row * p.ksc_pitch, dst + STG_NOPE + wu * KPW * 16, (1ull << KPW) - 1ull);
         } else {
             dma16(p.kr + (size_t)row * p.kr_pitch + 16 * (l & 7),
                   dst + STG_NOPE + STG_SCALE + (wu * KPW + 8 * (k - KPW / 2 - 1)) * (DR * 2));
@@ -377,11 +401,11 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * p.kr_pitch + 16 * (e & 7));
         }
     };
-    // De-quantisation of a staged tile, one eighth ("piece") at a time: fetch_piece reads the staged
-    // bytes into a few registers, emit_half de-quantises one half of them into the tile buffer.  The loop
-    // spreads the sixteen halves over its seventeen groups of four matrix products, each piece fetched
-    // one group before its first half is used, so that neither the LDS latency nor the vector
-    // instructions (about three per product) hold the matrix pipeline up.
+    // De-quantisation of a staged tile, one eighth ("piece") at a time: fetch_piece reads the staged bytes
+    // (eight per key and lane) and the key's scale into a few registers; emit_step (below) converts a quarter
+    // of one half of them -- the lower four bytes are half 0, the upper four half 1, which also stores the
+    // eight channels: the wave's 64 lanes write the 1024 contiguous bytes of the key's row in the tile
+    // buffer (tile = 0 or 1).  Each piece is fetched a few products before its first half is converted.
     constexpr int PER = (KPW + 7) / 8;             // keys of this wave per piece
     u32x2 praw[2][QUANT ? PER : 1], plow[QUANT ? PER : 1];
     float pbias[QUANT ? PER : 1];
@@ -393,25 +417,6 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             if (i < KPW) {
                 praw[piece & 1][q] = *reinterpret_cast<const u32x2 *>(pool_b + fetch_off + (slot * STG_BYTES + i * DN));
                 psc[piece & 1][q] = *reinterpret_cast<const float *>(pool_b + scale_off + (slot * STG_BYTES + i * 16));
-            }
-        }
-    };
-    // tile = 0 or 1: which of the two tile buffers.  Half 0 converts the lower four bytes, half 1 the upper
-    // four and stores the eight channels (the wave's 64 lanes: 1024 contiguous bytes of the key's row).
-    auto emit_half = [&](const int tile, const int piece, const int hf) {
-#pragma unroll
-        for (int q = 0; q < PER; ++q) {
-            const int i = piece * PER + q;
-            if (i < KPW) {
-                if (hf == 0) pbias[q] = -128.0f * psc[piece & 1][q];
-                const u32x2 c = dequant4(praw[piece & 1][q][hf], psc[piece & 1][q], pbias[q]);
-                if (hf == 0) {
-                    plow[q] = c;
-                } else {
-                    u32x4 v;
-                    v[0] = plow[q][0], v[1] = plow[q][1], v[2] = c[0], v[3] = c[1];
-                    *reinterpret_cast<u32x4 *>(pool_b + emit_off + (tile * KT * PITCH * 2 + i * PITCH * 2)) = v;
-                }
             }
         }
     };
@@ -434,42 +439,82 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
         }
     };
-    // what group u = 0..16 of a tile's products does for the next tile, before and after its products
-    // ... and for the tile after the next: its requests, REQ_PER_GROUP in each of the groups 1.., the cache
-    // row numbers read one group earlier (issued all at once the requests of the four waves queue up at
-    // the address unit for several hundred cycles; spread out they pass under the products)
-    constexpr int REQ_PER_GROUP = (DMA_PER_TILE + 15) / 16;
-    int srow[REQ_PER_GROUP];
-    auto group_pre = [&](const int u, const int slot, const int kt2, const int slot2) {
-        if (!QUANT) return;
-        if (u == 1) {
-            // the next tile's requests went out during the previous tile's products; the wait for the last
-            // of them comes after this tile's first products have been issued
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            asm volatile("" ::: "memory");
-        }
-        if (u % 2 == 1 && u / 2 < 8) fetch_piece(u / 2, slot);
-        if (u == 15) fetch_rope(slot);
-#pragma unroll
-        for (int j = 0; j < REQ_PER_GROUP; ++j) {
-            const int k = (u - 1) * REQ_PER_GROUP + j;
-            if (u >= 1 && k < DMA_PER_TILE) stage_request(slot2, k, srow[j]);
-        }
-#pragma unroll
-        for (int j = 0; j < REQ_PER_GROUP; ++j) {
-            const int k = u * REQ_PER_GROUP + j;
-            if (k < DMA_PER_TILE) srow[j] = stage_row(kt2, k);
+    // What product m = 0..67 of a tile (36 of S^T, then 32 of O^T) carries in its shadow for the following
+    // tiles.  A matrix product occupies the pipe for 32 clocks and a wave has one instruction stream: about
+    // four other instructions ride under a product for free, each further one costs about five clocks, and a
+    // product issued right behind another one wastes its shadow.  So the work is dealt out per product and
+    // every product ends with a scheduling barrier, which keeps the compiler from bunching it.  With
+    // u = m / 4 and e = m % 4:
+    //   m < 2 + DMA_PER_TILE   request m-2 of the tile after the next, its cache row numbers read from the row
+    //            table two products earlier: the requests go out under the tile's first products, which carry
+    //            nothing else, so that the last of them has nearly a whole tile's time to land (spread over
+    //            the tile they were still in flight when the next tile wanted them; all at once the requests
+    //            of the four waves queue up at the address unit for several hundred cycles)
+    //   e == 0   u odd: piece u/2 of the staged next tile is fetched from the staging ring (u == 1 first
+    //            waits for that tile's requests, all but the two just issued: requests complete in order);
+    //            u == 15: its rope piece
+    //   every e  a quarter of the de-quantisation of half u-2 of the next tile, about three vector
+    //            instructions per key of the wave's piece (the last four products carry halves 14 and 15)
+    static_assert(DMA_PER_TILE >= 2 && DMA_PER_TILE + 2 <= KSTEPS + 2 * DVB, "one request per product");
+    int srow[2];
+    // one key's dword at a time: step t = 0 .. 4*PER-1 of a half is quarter t%4 of the dword of key t/4
+    uint32_t dq_v = 0, dq_c = 0;
+    float dq_a = 0.f, dq_b = 0.f;
+    auto emit_step = [&](const int tile, const int h, const int t) {
+        const int piece = h / 2, hf = h % 2, q = t / 4, e = t % 4;
+        const int i = piece * PER + q;
+        if (i >= KPW) return;
+        const float sc = psc[piece & 1][q];
+        if (e == 0) {
+            if (hf == 0) pbias[q] = -128.0f * sc;
+            dq_v = praw[piece & 1][q][hf] ^ 0x80808080u;
+            dq_a = (float)(dq_v & 0xffu);
+            dq_b = (float)((dq_v >> 8) & 0xffu);
+        } else if (e == 1) {
+            dq_c = pack_bf16x2(__builtin_fmaf(dq_a, sc, pbias[q]), __builtin_fmaf(dq_b, sc, pbias[q]));
+            dq_a = (float)((dq_v >> 16) & 0xffu);
+        } else if (e == 2) {
+            dq_b = (float)(dq_v >> 24);
+            dq_a = __builtin_fmaf(dq_a, sc, pbias[q]);
+        } else {
+            const uint32_t c1 = pack_bf16x2(dq_a, __builtin_fmaf(dq_b, sc, pbias[q]));
+            if (hf == 0) {
+                plow[q][0] = dq_c, plow[q][1] = c1;
+            } else {
+                u32x4 v;
+                v[0] = plow[q][0], v[1] = plow[q][1], v[2] = dq_c, v[3] = c1;
+                *reinterpret_cast<u32x4 *>(pool_b + emit_off + (tile * KT * PITCH * 2 + i * PITCH * 2)) = v;
+            }
         }
     };
-    auto group_post = [&](const int u, const int tile) {
-        if (QUANT) {
-            if (u >= 2) emit_half(tile, (u - 2) / 2, (u - 2) % 2);
-            if (u == 16) {
-                emit_half(tile, 7, 1);
-                emit_rope(tile);
+    auto slot_work = [&](const int m, const int tile, const int slot, const int kt2, const int slot2) {
+        const int u = m / 4, e = m % 4;
+        if (!QUANT) {
+            if (m == KSTEPS) emit_rope(tile);
+            return;
+        }
+        if (m == 4) {
+            // the staged next tile has landed: everything but the two requests of products 2 and 3
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(2));
+            asm volatile("" ::: "memory");
+        }
+        if (m >= 2 && m - 2 < DMA_PER_TILE) stage_request(slot2, m - 2, srow[m & 1]);
+        if (m < DMA_PER_TILE) srow[m & 1] = stage_row(kt2, m);
+        if (e == 0) {
+            if (u % 2 == 1 && u / 2 < 8) fetch_piece(u / 2, slot);
+            if (u == 15) fetch_rope(slot);
+        }
+        if (u >= 2 && u < 16) {
+#pragma unroll
+            for (int j = 0; j < PER; ++j) emit_step(tile, u - 2, e * PER + j);
+        }
+        if (u == 16) {                      // the last four products carry halves 14 and 15
+#pragma unroll
+            for (int j = 0; j < 2 * PER; ++j) {
+                const int idx = e * 2 * PER + j;
+                emit_step(tile, 14 + idx / (4 * PER), idx % (4 * PER));
             }
-        } else if (u == KSTEPS / 4) {
-            emit_rope(tile);
+            if (e == 3) emit_rope(tile);
         }
     };
     // the first tile has nothing to hide behind: its staged bytes are fetched in batches of eight keys,
@@ -556,23 +601,17 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         f32x16 s;
         {
             const uint16_t *arow = cur_tile + tile_row_of(col) * PITCH + 8 * half;
-            bf16x8 fa[2][4];
+            // operand reads run four products ahead, in a ring of eight fragments
+            bf16x8 fa[8];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) fa[0][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * e);
+            for (int e = 0; e < 4; ++e) fa[e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * e);
 #pragma unroll
-            for (int g = 0; g < KSTEPS / 4; ++g) {
-                group_pre(g, (it + 1) & 1, kt + 2 * KT, it & 1);
-                if (g + 1 < KSTEPS / 4) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        fa[(g + 1) & 1][e] = *reinterpret_cast<const bf16x8 *>(arow + 16 * (4 * (g + 1) + e));
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (g == 0 && e == 0) s_mfma_first(s, fa[0][0], qf[0]);
-                    else s_mfma(s, fa[g & 1][e], qf[4 * g + e]);
-                }
-                group_post(g, (it + 1) & 1);
+            for (int m = 0; m < KSTEPS; ++m) {
+                if (m == 0) s_mfma_first(s, fa[0], qf[0]);
+                else s_mfma(s, fa[m & 7], qf[m]);
+                __builtin_amdgcn_sched_barrier(0);          // the product leads its slot
+                if (m + 4 < KSTEPS) fa[(m + 4) & 7] = *reinterpret_cast<const bf16x8 *>(arow + 16 * (m + 4));
+                slot_work(m, (it + 1) & 1, (it + 1) & 1, kt + 2 * KT, it & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -614,22 +653,19 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             AccLoop<0, DVB>::scale(o, alpha);
             valu_to_mfma_fence();
         }
-        bf16x8 pf[2];
-        auto pack_p = [&](const int kk) {
-            u32x4 pk;
+        // P^T of the first sixteen keys is packed here; the exponentials of the other sixteen (needed by the
+        // second half of the PV products only), their packing and the row sum are dealt out over the first
+        // thirteen PV products
+        u32x4 pk0, pk1;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) pk[e] = pack_bf16x2(s[8 * kk + 2 * e], s[8 * kk + 2 * e + 1]);
-            pf[kk] = __builtin_bit_cast(bf16x8, pk);
-        };
-        pack_p(0);
-        auto softmax_tail = [&](const int part) {
-#pragma unroll
-            for (int r = 8 + 4 * part; r < 12 + 4 * part; ++r) {
-                s[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc_log2, -m_new));
-                lsum += s[r];
-            }
-            if (part == 1) {
-                pack_p(1);
+        for (int e = 0; e < 4; ++e) pk0[e] = pack_bf16x2(s[2 * e], s[2 * e + 1]);
+        auto softmax_slice = [&](const int mp) {
+            if (mp < 8) {
+                s[8 + mp] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[8 + mp], sc_log2, -m_new));
+                lsum += s[8 + mp];
+            } else if (mp < 12) {
+                pk1[mp - 8] = pack_bf16x2(s[8 + 2 * (mp - 8)], s[8 + 2 * (mp - 8) + 1]);
+            } else if (mp == 12) {
                 float lo, hi;
                 both_halves(lsum, lo, hi);
                 lsum = lo + hi;
@@ -637,37 +673,29 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
         };
 
-        // ---- O^T += V^T . P^T: product m = 16*kk + dvb, V^T reads one group of four products ahead;
-        // interleaved with the de-quantisation of the next tile into the other buffer
+        // ---- O^T += V^T . P^T: product mp = 16*kk + dvb, V^T reads four products ahead in a ring of eight;
+        // each product carries its share of the work for the following tiles (slot_work)
         {
             const uint16_t *vbase = cur_tile + (half + 4 * ((l & 15) >> 2)) * PITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
-            s16x4 va[2][4][2];
+            s16x4 va[8][2];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                va[0][e][0] = lds_read_tr16(vbase + 32 * e);
-                va[0][e][1] = lds_read_tr16(vbase + 32 * e + 2 * PITCH);
+                va[e][0] = lds_read_tr16(vbase + 32 * e);
+                va[e][1] = lds_read_tr16(vbase + 32 * e + 2 * PITCH);
             }
 #pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                group_pre(KSTEPS / 4 + g, (it + 1) & 1, kt + 2 * KT, it & 1);
-                if (g + 1 < 8) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int m = 4 * (g + 1) + e;
-                        const uint16_t *a0 = vbase + (16 * (m >> 4)) * PITCH + 32 * (m & 15);
-                        va[(g + 1) & 1][e][0] = lds_read_tr16(a0);
-                        va[(g + 1) & 1][e][1] = lds_read_tr16(a0 + 2 * PITCH);
-                    }
+            for (int mp = 0; mp < 2 * DVB; ++mp) {
+                const s16x8 a = __builtin_shufflevector(va[mp & 7][0], va[mp & 7][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                acc_mfma(o[mp & 15], __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, mp < DVB ? pk0 : pk1));
+                __builtin_amdgcn_sched_barrier(0);          // the product leads its slot
+                if (mp + 4 < 2 * DVB) {
+                    const int m2 = mp + 4;
+                    const uint16_t *a0 = vbase + (16 * (m2 >> 4)) * PITCH + 32 * (m2 & 15);
+                    va[m2 & 7][0] = lds_read_tr16(a0);
+                    va[m2 & 7][1] = lds_read_tr16(a0 + 2 * PITCH);
                 }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int m = 4 * g + e;
-                    const s16x8 a = __builtin_shufflevector(va[g & 1][e][0], va[g & 1][e][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                    acc_mfma(o[m & 15], __builtin_bit_cast(bf16x8, a), pf[m >> 4]);
-                }
-                if (g < 2) softmax_tail(g);
-                // a sixteenth of the next tile's de-quantisation rides in the shadow of these products
-                group_post(KSTEPS / 4 + g, (it + 1) & 1);
+                softmax_slice(mp);
+                slot_work(KSTEPS + mp, (it + 1) & 1, (it + 1) & 1, kt + 2 * KT, it & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
