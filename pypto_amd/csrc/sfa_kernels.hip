@@ -73,6 +73,13 @@ __device__ __forceinline__ void acc_mfma(f32x16 &acc, const bf16x8 a, const bf16
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
 }
 
+// First product into an O^T block: starts from zero, so the 256 accumulation registers need no clearing
+// (256 writes in front of the key loop otherwise).
+__device__ __forceinline__ void acc_mfma_first(f32x16 &acc, const bf16x8 a, const bf16x8 b)
+{
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b));
+}
+
 // S^T accumulator: kept in architectural registers by construction.  Left to the compiler it shares the
 // first sixteen accumulation registers with the first O^T block, which is then copied out and back
 // around every tile.  First product of a chain starts from zero; the chain is dependent products on one
@@ -325,12 +332,16 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         }
     }
 
+    // int8 cache: the first tile's products start the accumulators from zero (acc_mfma_first); they are
+    // cleared beforehand only when there is no first tile, or for the bf16 cache's single-bodied loop
     f32x16 o[DVB];
+    if (!QUANT || k_begin >= k_end) {
 #pragma unroll
-    for (int i = 0; i < DVB; ++i)
+        for (int i = 0; i < DVB; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-    valu_to_mfma_fence();
+            for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+        valu_to_mfma_fence();
+    }
     float m_run = -INFINITY;   // reference max, log2 domain
     float l_run = 0.f;         // running sum of exp2(s - m_run)
 
@@ -589,8 +600,9 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // One tile.  For the int8 cache the parity of the tile number is a compile-time constant (the loop
     // below runs two tiles per trip), so every LDS address in here is a per-lane base plus an immediate
     // offset.
-    auto tile_step = [&](auto parity, const int kt) __attribute__((always_inline)) {
+    auto tile_step = [&](auto parity, auto first_tag, const int kt) __attribute__((always_inline)) {
         const int it = parity;
+        constexpr bool FIRST = decltype(first_tag)::value;     // the split's first tile (int8 cache only)
         const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
         uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
         // next tile (or a padding tile) of the bf16 cache, the tile after it of the int8 cache: in flight
@@ -648,7 +660,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             lsum += s[r];
         }
         m_run = m_new;
-        if (__builtin_expect(__any(rescale), 0)) {               // rare: laid out away from the loop body
+        if (!FIRST && __builtin_expect(__any(rescale), 0)) {     // rare: laid out away from the loop body
             mfma_to_valu_fence();
             AccLoop<0, DVB>::scale(o, alpha);
             valu_to_mfma_fence();
@@ -686,7 +698,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 #pragma unroll
             for (int mp = 0; mp < 2 * DVB; ++mp) {
                 const s16x8 a = __builtin_shufflevector(va[mp & 7][0], va[mp & 7][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                acc_mfma(o[mp & 15], __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, mp < DVB ? pk0 : pk1));
+                if (FIRST && mp < DVB) acc_mfma_first(o[mp], __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, pk0));
+                else acc_mfma(o[mp & 15], __builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, mp < DVB ? pk0 : pk1));
                 __builtin_amdgcn_sched_barrier(0);          // the product leads its slot
                 if (mp + 4 < 2 * DVB) {
                     const int m2 = mp + 4;
@@ -704,13 +717,17 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     };
     if constexpr (QUANT) {
         // an odd number of tiles is rounded up: the extra tile holds padding rows only, all of them masked
-        for (int kt = k_begin; kt < k_end; kt += 2 * KT) {
-            tile_step(std::integral_constant<int, 0>{}, kt);
-            tile_step(std::integral_constant<int, 1>{}, kt + KT);
+        if (k_begin < k_end) {
+            tile_step(std::integral_constant<int, 0>{}, std::true_type{}, k_begin);
+            tile_step(std::integral_constant<int, 1>{}, std::false_type{}, k_begin + KT);
+        }
+        for (int kt = k_begin + 2 * KT; kt < k_end; kt += 2 * KT) {
+            tile_step(std::integral_constant<int, 0>{}, std::false_type{}, kt);
+            tile_step(std::integral_constant<int, 1>{}, std::false_type{}, kt + KT);
         }
     } else {
         int it = 0;
-        for (int kt = k_begin; kt < k_end; kt += KT, ++it) tile_step(it & 1, kt);
+        for (int kt = k_begin; kt < k_end; kt += KT, ++it) tile_step(it & 1, std::false_type{}, kt);
     }
     if (QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);      // the padding tiles' requests have landed: the pool is quiet
 
