@@ -817,8 +817,10 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 
 // Merges the key splits of one query row: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - m)
 // and O_s the split's normalised fp16 partial (all zeros for an empty split, whose weight is zero).
-// One thread per (row, head, 8 value channels); splits are taken eight at a time with all their loads
-// in flight together.
+// One thread per (row, head, 8 value channels); splits are taken NS at a time with all their loads in flight
+// together (NS = 2, 4 or 8: the smallest that covers the launch's splits in one trip, so that a row of two
+// splits does not load its last split seven times over).
+template <int NS>
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
 {
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -832,27 +834,27 @@ __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
     const f32x2 *ml = reinterpret_cast<const f32x2 *>(p.part_ml);
 
     float m = -INFINITY;
-    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
-        f32x2 v[8];
+    for (int s0 = 0; s0 < p.nsplit; s0 += NS) {
+        f32x2 v[NS];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = ml[prow0 + (size_t)(s0 + e < p.nsplit ? s0 + e : p.nsplit - 1) * p.NQ];
+        for (int e = 0; e < NS; ++e) v[e] = ml[prow0 + (size_t)(s0 + e < p.nsplit ? s0 + e : p.nsplit - 1) * p.NQ];
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
+        for (int e = 0; e < NS; ++e)
             if (v[e][1] > 0.f) m = fmaxf(m, v[e][0]);
     }
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float wsum = 0.f;
-    for (int s0 = 0; s0 < p.nsplit; s0 += 8) {
-        f32x2 v[8];
-        f16x8 hv[8];
+    for (int s0 = 0; s0 < p.nsplit; s0 += NS) {
+        f32x2 v[NS];
+        f16x8 hv[NS];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < NS; ++e) {
             const size_t prow = prow0 + (size_t)(s0 + e < p.nsplit ? s0 + e : p.nsplit - 1) * p.NQ;
             v[e] = ml[prow];
             hv[e] = *reinterpret_cast<const f16x8 *>(p.part_o + prow * DN + 8 * c8);
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < NS; ++e) {
             const bool live = s0 + e < p.nsplit && v[e][1] > 0.f;
             const float wgt = live ? v[e][1] * __builtin_amdgcn_exp2f(v[e][0] - m) : 0.f;
 #pragma unroll
@@ -890,7 +892,10 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
     if (e != hipSuccess) return e;
     if (p.nsplit > 1) {
         const size_t total = (size_t)p.T * p.NQ * (DN / 8);
-        hipLaunchKernelGGL(sfa_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
+        const dim3 cgrid((unsigned)((total + 255) / 256));
+        if (p.nsplit <= 2) hipLaunchKernelGGL(sfa_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
+        else if (p.nsplit <= 4) hipLaunchKernelGGL(sfa_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL(sfa_combine_kernel<8>, cgrid, dim3(256), 0, stream, p);
         e = hipGetLastError();
     }
     return e;
