@@ -332,10 +332,10 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         }
     }
 
-    // int8 cache: the first tile's products start the accumulators from zero (acc_mfma_first); they are
-    // cleared beforehand only when there is no first tile, or for the bf16 cache's single-bodied loop
+    // the first tile's products start the accumulators from zero (acc_mfma_first); they are cleared beforehand
+    // only when there is no first tile
     f32x16 o[DVB];
-    if (!QUANT || k_begin >= k_end) {
+    if (k_begin >= k_end) {
 #pragma unroll
         for (int i = 0; i < DVB; ++i)
 #pragma unroll
@@ -501,7 +501,26 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     auto slot_work = [&](const int m, const int tile, const int slot, const int kt2, const int slot2) {
         const int u = m / 4, e = m % 4;
         if (!QUANT) {
-            if (m == KSTEPS) emit_rope(tile);
+            // bf16 cache: the next tile's rows go straight into the other tile buffer, one request per key of
+            // this wave under the tile's first products, the rope pieces through registers
+            constexpr int NREQ = KT / NW;
+            constexpr int ROPE_LOAD_AT = NREQ > KSTEPS ? NREQ : KSTEPS;     // held in registers for twelve products
+            const int kt1 = kt2 - KT;
+            uint16_t *buf = tile ? tile1 : tile0;
+            if (m < NREQ) {
+                const int row = rows_lds[(kt1 - k_begin) + wu * NREQ + m];
+                dma16(p.kn + (size_t)row * p.kn_pitch + 16 * l,
+                      (uint32_t)(uintptr_t)(lds_byte_t *)buf + (uint32_t)((wu * NREQ + m) * PITCH * 2));
+            }
+            if (m == ROPE_LOAD_AT) {
+#pragma unroll
+                for (int i = 0; i < RP; ++i) {
+                    const int e2 = tid + i * NW * 64;
+                    const int row = rows_lds[(kt1 - k_begin) + (e2 >> 3)];
+                    rrope[i] = *reinterpret_cast<const u32x4 *>(p.kr + (size_t)row * p.kr_pitch + 16 * (e2 & 7));
+                }
+            }
+            if (m == ROPE_LOAD_AT + 12) emit_rope(tile);
             return;
         }
         if (m == 4) {
@@ -604,11 +623,6 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         const int it = parity;
         constexpr bool FIRST = decltype(first_tag)::value;     // the split's first tile (int8 cache only)
         const uint16_t *cur_tile = (it & 1) ? tile1 : tile0;
-        uint16_t *nxt_tile = (it & 1) ? tile0 : tile1;
-        // next tile (or a padding tile) of the bf16 cache, the tile after it of the int8 cache: in flight
-        // during the products
-        if (!QUANT) issue_loads(kt + KT, nxt_tile);
-
         // ---- S^T = K . Q^T, LDS reads running one group of four contraction steps ahead
         f32x16 s;
         {
@@ -715,7 +729,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         if (!QUANT) __builtin_amdgcn_s_waitcnt(0x0F70); // this wave's direct requests into the next tile have landed
         __syncthreads();
     };
-    if constexpr (QUANT) {
+    {
         // an odd number of tiles is rounded up: the extra tile holds padding rows only, all of them masked
         if (k_begin < k_end) {
             tile_step(std::integral_constant<int, 0>{}, std::true_type{}, k_begin);
@@ -725,11 +739,8 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             tile_step(std::integral_constant<int, 0>{}, std::false_type{}, kt);
             tile_step(std::integral_constant<int, 1>{}, std::false_type{}, kt + KT);
         }
-    } else {
-        int it = 0;
-        for (int kt = k_begin; kt < k_end; kt += KT, ++it) tile_step(it & 1, std::false_type{}, kt);
     }
-    if (QUANT) __builtin_amdgcn_s_waitcnt(0x0F70);      // the padding tiles' requests have landed: the pool is quiet
+    __builtin_amdgcn_s_waitcnt(0x0F70);                 // the padding tiles' requests have landed: the pool is quiet
 
     // ---- epilogue.  Lane (head, half) holds value channels 32*dvb + 8*(r/4) + 4*half + r%4 of its head;
     // written from there each store instruction would touch 32 rows with 8 bytes each.  Each wave
