@@ -520,7 +520,7 @@ def main():
                      "frac": achieved_tflops / PEAK_BF16_TFLOPS,
                      "traffic": measured_traffic(TRAFFIC_FILE, "traffic_bytes_per_step", lib_version,
                                                  {"key_splits": key_splits}),
-                     "kernel": "sfa_decode_kernel<4> + sfa_combine_kernel (one step)",
+                     "kernel": "sfa_decode_kernel<4> + sfa_combine_kernel<8> (one step)",
                      "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "flops_per_launch": flops},
         "roofline_hbm": {"bound": "hbm", "achieved": achieved_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": achieved_gbs / PEAK_HBM_GBS, "bytes_per_launch": byt},
