@@ -426,7 +426,8 @@ def main():
         pypto_amd.sparse_attention_antiquant_d(sfa_d.query_nope, sfa_d.query_rope, packed, sel[i % ROT],
                                                sfa_d.block_table, sfa_d.kv_act_seqs, out_p, NQ, 1,
                                                sfa.softmax_scale, K, 128, sfa.max_blocknum_perbatch, None)
-    _, packed_avg_ms, _ = time_events(packed_step, max(args.steps // 2, 5), 20, torch)
+    # timed like the steps above, and after as many settling steps: packing the cache left the device idle
+    packed_avg_ms = time_batch(packed_step, max(args.steps // 2, 5), SETTLE_STEPS, torch)
     sfa_step(0)
     packed_step(0)
     torch.cuda.synchronize()
