@@ -15,6 +15,7 @@ constexpr int MLAP_MAX_XGROUPS = 32; // h <= 32 * 8 * 64 = 16384
 constexpr int MLAP_MAX_QLORA = 1536;
 constexpr int QPROJ_KSPLIT_HOST = 4; // partial sums of the int8 projection (prolog_common.h: QPROJ_KSPLIT)
 constexpr int MLAP_XTOK = 8;         // tokens per job of the first and of the last kernel
+constexpr int MLAP_MFMA_MIN_TOKENS = 64;   // from here on the first launch sums on the matrix cores (unless absorb_exact)
 
 struct MlapParams {
     const uint16_t *x;            // [T, h] bf16
@@ -42,7 +43,8 @@ struct MlapParams {
     float eps_cq, eps_ckv;
     int absorb_exact;             // 1: the product with w_uk as fixed-order fp32 sums (bit-reproducible against the
                                   // sequential statement); 0: on the matrix cores (bf16 x bf16 exact, fp32 sums in the
-                                  // cores' own order: differs in the last bit of some results)
+                                  // cores' own order: differs in the last bit of some results), and from
+                                  // MLAP_MFMA_MIN_TOKENS tokens on the sums over the hidden axis as well
 };
 
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);

@@ -118,6 +118,34 @@ def test_mla_prolog_prefill_t512():
     assert_exact(run_op(inp, (1e-5, 1e-5), prefill=True), ref, "t_512 prefill")
 
 
+def test_mla_prolog_prefill_t512_matrix_core_sums_default():
+    """The operator's default from 64 tokens on: the sums over the hidden axis run on the matrix cores as well
+    (same exact products, the cores' own summation order), so the int8 latents may differ by one step where the
+    sequential sums land next to a rounding boundary.  Held to the reference's acceptance rule for every output
+    (deepseekv32_mla_prolog_quant.py:668-692) against the sequential statement; a short-h shape with ragged
+    token tiles and a half-empty chunk split rides along."""
+    from pypto_amd import mla_prolog_quant_impl as impl
+    impl.EXACT_ABSORB = False
+    for b, s1, act, kw in ((1, 512, [4096], {}), (3, 50, [700] * 3, dict(h=192, q_lora_rank=512, n_heads=2))):
+        inp = gen_mla_prolog_inputs(b, s1, act, seed=41 + b, **kw)
+        ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+        got = run_op(inp, (1e-5, 1e-5), prefill=True)
+        rows = inp.cache_index.numpy()
+        dq = np.abs(got["q_norm"].astype(np.int32) - ref["q_norm"].astype(np.int32))
+        assert dq.max() <= 1 and (dq != 0).mean() <= 0.01
+        assert np.abs(got["q_norm_scale"] - ref["q_norm_scale"]).max() <= 2.5e-5 + 0.005 * np.abs(ref["q_norm_scale"]).max()
+        for name in ("query_nope", "query_rope"):
+            g, r = got[name], ref[name]
+            assert (np.abs(g - r) > 0.005 + 0.0078125 * np.abs(r)).mean() <= 0.005, name
+        gk, rk = got["kv_cache"].reshape(-1, 512)[rows].astype(np.int32), ref["kv_cache"].reshape(-1, 512)[rows].astype(np.int32)
+        assert np.abs(gk - rk).max() <= 1 and (gk != rk).mean() <= 0.01
+        gr, rr = got["kr_cache"].reshape(-1, 64)[rows], ref["kr_cache"].reshape(-1, 64)[rows]
+        assert np.abs(gr - rr).max() <= 1e-4 + 0.0078125 * np.abs(rr).max()
+        gs, rs = got["k_scale_cache"].reshape(-1, 4)[rows], ref["k_scale_cache"].reshape(-1, 4)[rows]
+        assert np.abs(gs - rs).max() <= 2.5e-5 + 0.005 * np.abs(rs).max()
+        print(f"t={b * s1}: q_norm entries off by one {float((dq != 0).mean()):.5f}, latent entries off by one {float((gk != rk).mean()):.5f}", flush=True)
+
+
 def test_mla_prolog_separate_cache_output_skipped_indices_and_repeatability():
     inp = gen_mla_prolog_inputs(2, 2, [300, 129], seed=5, h=256, q_lora_rank=512, n_heads=4)
     inp.cache_index[1] = -1
