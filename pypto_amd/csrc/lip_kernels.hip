@@ -164,6 +164,12 @@ __global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const
     if (qwave && w == 0) q_pair_store<HS>(qp, lip_smem, job, l, acc);
 }
 
+__global__ __launch_bounds__(256) void lip_qproj_prefill_kernel(const QProj p, const int njobs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[QPF_LDS];
+    q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second launch: prolog_finish.h.
 __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
@@ -180,7 +186,16 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
 {
     const int steps = p.q_lora / LIP_KSPLIT / 32;
     const int tblocks = (p.T + 31) / 32;
-    const int q_jobs = p.n_heads * LIP_KSPLIT * tblocks;
+    const bool unsplit = qproj_splits(p.T) == 1;      // prefill sizes: the query projection as a launch of its own
+    const int q_jobs = unsplit ? 0 : p.n_heads * LIP_KSPLIT * tblocks;
+    if (unsplit) {
+        if (p.q_lora % (32 * QPF_STEPS)) return hipErrorInvalidValue;
+        const QProj qp = {p.q_norm, p.w_qb, p.qpart, p.T, p.q_lora, p.n_heads};
+        const int njobs = q_prefill_jobs(qp);
+        hipLaunchKernelGGL(lip_qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     const int x_jobs = 2 * (p.h / LIP_XBLOCK) * ((p.T + XTOK - 1) / XTOK);
     // enough workgroups that each hidden-axis wave gets about one job, never fewer than the query jobs
     int wgs = (x_jobs + LIN_XWAVES - 1) / LIN_XWAVES;

@@ -428,6 +428,12 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njo
     }
 }
 
+__global__ __launch_bounds__(256) void qproj_prefill_kernel(const QProj p, const int njobs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[QPF_LDS];
+    q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Last launch: prolog_finish.h.
 __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
@@ -461,6 +467,12 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128};
+    if (qproj_splits(p.T) == 1) {
+        if (p.q_lora % (32 * QPF_STEPS)) return hipErrorInvalidValue;
+        const int njobs = q_prefill_jobs(qp);
+        hipLaunchKernelGGL(qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+        return hipGetLastError();
+    }
     const int qjobs = qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);
     // as many workgroups as fit at once (by their LDS), every one with the same number of jobs where possible
     const int steps = p.q_lora / QPROJ_KSPLIT / 32;

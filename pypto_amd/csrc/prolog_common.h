@@ -8,11 +8,15 @@ namespace pto {
 namespace {
 
 constexpr int QPROJ_KSPLIT = 4;     // jobs that share the reduction axis of the int8 projection
+constexpr int QPROJ_PREFILL_TOKENS = 64;   // from this many tokens on the projection runs unsplit (q_prefill_body)
+
+// partial sums per output of the int8 projection at T tokens
+__host__ __device__ inline int qproj_splits(const int T) { return T >= QPROJ_PREFILL_TOKENS ? 1 : QPROJ_KSPLIT; }
 
 struct QProj {
     const int8_t *q_norm;   // [T, q_lora]
     const int8_t *w;        // [q_lora, 128 * nslabs], row-major
-    int32_t *part;          // [QPROJ_KSPLIT, T, 128 * nslabs]
+    int32_t *part;          // [qproj_splits(T), T, 128 * nslabs]
     int T, q_lora, nslabs;
 };
 
@@ -93,17 +97,15 @@ __device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const i
     }
 }
 
-// one 32-row step of the product from the wave's region
-template <int HS>
-__device__ __forceinline__ void q_step(const uint8_t *region, const int s, const int l, i32x16 (&acc)[4])
+// one 32-row step of the product: rows 32s.. of the tile, token operands of step s at tok + 1024 s
+__device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *tok, const int s, const int l, i32x16 (&acc)[4])
 {
-    constexpr int KH = HS * 32;
-    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(region);
+    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(tile);
     const int rd = (16 * (l >> 5)) * 32 + (l & 31);     // dword index of this lane's first row of a step
     uint32_t d[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
-    const i32x4 b = *reinterpret_cast<const i32x4 *>(region + KH * 128 + 1024 * s + 16 * l);
+    const i32x4 b = *reinterpret_cast<const i32x4 *>(tok + 1024 * s + 16 * l);
     i32x4 a[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -116,6 +118,12 @@ __device__ __forceinline__ void q_step(const uint8_t *region, const int s, const
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+}
+// the same from a wave's region of a split job
+template <int HS>
+__device__ __forceinline__ void q_step(const uint8_t *region, const int s, const int l, i32x16 (&acc)[4])
+{
+    q_step_at(region, region + HS * 32 * 128, s, l, acc);
 }
 
 // A single job: issue, then every step as soon as its four requests have landed (requests complete
@@ -176,6 +184,77 @@ __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const 
         i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
         red[r * 64 + l] = v;
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The projection at prefill sizes (T >= QPROJ_PREFILL_TOKENS): one workgroup of four waves per (slab of 128
+// columns, block of 128 tokens) walks the whole reduction axis in chunks of 128 rows, so a weight tile is read
+// once per 128 tokens instead of once per 32 and no partial sums are left to add.  Wave w takes tokens 32w..32w+31
+// of the block; the chunk of the tile (16 KiB, shared) and each wave's token operands (4 KiB) travel by LDS-DMA into
+// one of two buffers, a chunk ahead of the products that read them.  Same products and lane layout as a split job.
+constexpr int QPF_STEPS = 4;                           // 32-row steps per chunk
+constexpr int QPF_TILE = QPF_STEPS * 32 * 128;
+constexpr int QPF_TOK = QPF_STEPS * 1024;
+constexpr int QPF_BUF = QPF_TILE + 4 * QPF_TOK;
+constexpr int QPF_LDS = 2 * QPF_BUF;                   // 64 KiB
+
+__host__ __device__ inline int q_prefill_jobs(const QProj &p) { return p.nslabs * ((p.T + 127) / 128); }
+
+// job: the blocks of a slab are neighbours in the job order
+__device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, uint8_t *lds)
+{
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ncols = p.nslabs * 128;
+    const int ttiles = (p.T + 127) / 128;
+    const int slab = job / ttiles;
+    const int t = (job % ttiles) * 128 + 32 * w + (l & 31);
+    const int nch = p.q_lora / (32 * QPF_STEPS);
+    const int8_t *tsrc = p.q_norm + (size_t)(t < p.T ? t : p.T - 1) * p.q_lora + 16 * (l >> 5);
+    const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * (l & 7);
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
+    auto issue = [&](const int c) {
+        const uint32_t buf = base + (c & 1) * QPF_BUF;
+#pragma unroll
+        for (int s = 0; s < QPF_STEPS; ++s) dma16(tsrc + c * (32 * QPF_STEPS) + 32 * s, buf + QPF_TILE + w * QPF_TOK + 1024 * s);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(wsrc + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
+    };
+    i32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+    issue(0);
+#pragma unroll 1
+    for (int c = 0; c < nch; ++c) {
+        if (c + 1 < nch) {
+            issue(c + 1);
+            VM_WAIT(QPF_STEPS + 4);
+        } else {
+            VM_WAIT(0);
+        }
+        __syncthreads();                               // every wave's share of chunk c has landed
+        const uint8_t *buf = lds + (c & 1) * QPF_BUF;
+#pragma unroll
+        for (int s = 0; s < QPF_STEPS; ++s) q_step_at(buf, buf + QPF_TILE + w * QPF_TOK, s, l, acc);
+        __syncthreads();                               // chunk c + 2 goes where chunk c was read
+    }
+    if (t < p.T) {
+        int32_t *dst = p.part + (size_t)t * ncols + slab * 128;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
+            const i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+            *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
+        }
+    }
+}
+// workgroup number -> job, so that the workgroups of a slab (consecutive jobs) run on one XCD (workgroups go round
+// the eight XCDs) and share its L2 copy of the weight tile
+__device__ __forceinline__ int q_prefill_job_of(const int wg, const int njobs)
+{
+    return (njobs & 7) == 0 ? (wg & 7) * (njobs >> 3) + (wg >> 3) : wg;
 }
 
 // Cross-lane exchanges without LDS traffic.  dpp_f32 reads another lane of the same row of 16;

@@ -12,6 +12,25 @@
 namespace pto {
 namespace {
 
+// the int8 projection's result for columns col, col + 1 of token t: its partial sums added
+__device__ __forceinline__ void part_sum2(const int32_t *part, const int T, const int t, const int ncols, const int col, int &s0, int &s1)
+{
+    if (qproj_splits(T) == 1) {
+        const int2 v = *reinterpret_cast<const int2 *>(part + (size_t)t * ncols + col);
+        s0 = v.x;
+        s1 = v.y;
+        return;
+    }
+    s0 = 0;
+    s1 = 0;
+#pragma unroll
+    for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
+        const int2 v = *reinterpret_cast<const int2 *>(part + ((size_t)kq * T + t) * ncols + col);
+        s0 += v.x;
+        s1 += v.y;
+    }
+}
+
 // ------------------------------------------------------------------------------ indexer prolog
 // rope on channels 0..63 (lanes 0..31 hold channels 2l, 2l+1); the rotation partner of channel i is
 // i+32 (negated) for i < 32 and i-32 otherwise: lane l ^ 16.  Results rounded to bf16.
@@ -122,13 +141,8 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
         const int t = live ? row / p.n_heads : 0;
         const int head = live ? row % p.n_heads : 0;
         const int col = head * LIP_DIM + 2 * l;
-        int s0 = 0, s1 = 0;
-#pragma unroll
-        for (int kq = 0; kq < LIP_KSPLIT; ++kq) {
-            const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + t) * ncols + col);
-            s0 += v.x;
-            s1 += v.y;
-        }
+        int s0, s1;
+        part_sum2(p.qpart, p.T, t, ncols, col, s0, s1);
         const float ts = p.q_norm_scale[t];
         const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
         const uint32_t rc = rope_coef(p.cos, t, l), rs = rope_coef(p.sin, t, l);
@@ -266,13 +280,8 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
         // nope part: lane l -> channels 2l, 2l+1
         {
             const int col = head * MLAP_QHEAD + 2 * l;
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
-                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + tt) * ncols + col);
-                s0 += v.x;
-                s1 += v.y;
-            }
+            int s0, s1;
+            part_sum2(p.qpart, p.T, tt, ncols, col, s0, s1);
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
             f32x2 av = {bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0])),
                         bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]))};
@@ -282,13 +291,8 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
         // rope part (first half-workgroup only): lane l < 32 -> channels 2l, 2l+1 = rotation partners l, 32+l
         if (half == 0 && l < 32 && t < p.T) {
             const int col = head * MLAP_QHEAD + MLAP_NOPE + 2 * l;
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
-                const int2 v = *reinterpret_cast<const int2 *>(p.qpart + ((size_t)kq * p.T + t) * ncols + col);
-                s0 += v.x;
-                s1 += v.y;
-            }
+            int s0, s1;
+            part_sum2(p.qpart, p.T, t, ncols, col, s0, s1);
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
             const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
             const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
