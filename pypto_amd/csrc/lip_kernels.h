@@ -46,5 +46,6 @@ hipError_t lip_launch(const LipParams &p, hipStream_t stream);
 // the first launch alone, and the number of query-row workgroups of the second (for the fused operator's last launch)
 hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream);
 int lip_finish_query_wgs(const LipParams &p);
+hipError_t lip_launch_finish(const LipParams &p, hipStream_t stream);   // the second launch alone
 
 }  // namespace pto

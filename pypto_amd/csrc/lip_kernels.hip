@@ -215,6 +215,11 @@ hipError_t lip_launch(const LipParams &p, hipStream_t stream)
 {
     hipError_t e = lip_launch_linear(p, stream);
     if (e != hipSuccess) return e;
+    return lip_launch_finish(p, stream);
+}
+
+hipError_t lip_launch_finish(const LipParams &p, hipStream_t stream)
+{
     const int q_wgs = lip_finish_query_wgs(p);
     hipLaunchKernelGGL(lip_finish_kernel, dim3((unsigned)(q_wgs + p.T)), dim3(64 * FIN_WAVES), 0, stream, p, q_wgs);
     return hipGetLastError();

@@ -51,5 +51,9 @@ hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
 // all launches but the last, and the number of workgroups of the last (for the fused operator's last launch)
 hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream);
 int mlap_finish_wgs(const MlapParams &p);
+// the last launch alone; at prefill sizes (mlap_finish_is_prefill) it has a form of its own that the fused operator
+// launches beside, not inside, its own last launch
+hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream);
+bool mlap_finish_is_prefill(const MlapParams &p);
 
 }  // namespace pto

@@ -442,7 +442,30 @@ __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
     mlap_finish_body(p, (int)blockIdx.x, lds);
 }
 
+__global__ __launch_bounds__(64 * FINP_WAVES) void mlap_finish_prefill_kernel(const MlapParams p, const int per)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[MLAP_FINP_LDS];
+    mlap_finish_prefill_body(p, (int)blockIdx.x, per, lds);
+}
+
 }  // namespace
+
+bool mlap_finish_is_prefill(const MlapParams &p) { return p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact; }
+
+hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream)
+{
+    if (mlap_finish_is_prefill(p)) {
+        // runs of up to 16 blocks of 32 tokens per workgroup, two runs at least so that 128 heads fill the chip
+        const int nblocks = (p.T + FINP_TOK - 1) / FINP_TOK;
+        int per = (nblocks + 1) / 2;
+        per = per > 16 ? 16 : per;
+        const int runs = (nblocks + per - 1) / per;
+        hipLaunchKernelGGL(mlap_finish_prefill_kernel, dim3((unsigned)(p.n_heads * runs)), dim3(64 * FINP_WAVES), 0, stream, p, per);
+    } else {
+        hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)mlap_finish_wgs(p)), dim3(256), 0, stream, p);
+    }
+    return hipGetLastError();
+}
 
 int mlap_finish_wgs(const MlapParams &p) { return p.n_heads * 2 * ((p.T + MLAP_XTOK - 1) / MLAP_XTOK); }
 
@@ -495,8 +518,7 @@ hipError_t mlap_launch(const MlapParams &p, hipStream_t stream)
 {
     hipError_t e = mlap_launch_front(p, stream);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)mlap_finish_wgs(p)), dim3(256), 0, stream, p);
-    return hipGetLastError();
+    return mlap_launch_finish(p, stream);
 }
 
 }  // namespace pto

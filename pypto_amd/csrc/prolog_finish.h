@@ -388,7 +388,127 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
             p.q_nope[((size_t)(t0 + t) * p.n_heads + head) * MLAP_KV + colbase + l] = (uint16_t)(pack_bf16x2(acc[t], 0.f) & 0xffffu);
 }
 
+// ------------------------------------------------------------------------ MLA prolog, prefill sizes
+// The same last stage for 64 tokens and more with the absorb product on the matrix cores: one workgroup of eight
+// waves per (head, run of `per` blocks of 32 tokens).  The head's whole w_uk (128 x 512 bf16, 128 KiB) is staged
+// once, wave w keeping the slice of output columns 64w..64w+63 in the layout of the decode form; then per block:
+// wave w de-quantises the query channels of tokens 4w..4w+3 (the projection is unsplit at these sizes) into one of two
+// bf16 operand buffers and rotates and stores their rope part, the loads of the next block go out, one barrier, and
+// 16 products per wave give 32 tokens x 64 columns.  A weight slice is read once per `per` blocks instead of once
+// per 8 tokens; each output has the bits of the decode form (same products, same order).
+constexpr int FINP_TOK = 32;
+constexpr int FINP_WAVES = 8;
+constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * MLAP_NOPE * 2;   // 147 456 bytes
+static_assert(MLAP_MFMA_MIN_TOKENS >= QPROJ_PREFILL_TOKENS, "the prefill form reads one partial sum per output");
 
+struct FinRaw {
+    int2 nope[4], rope[4];
+    float ts[4];
+    uint16_t c0[4], c1[4], s0[4], s1[4];
+};
+
+__device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, const int wg, const int per, uint8_t *lds)
+{
+    uint8_t *wsl = lds;
+    uint16_t(*abf)[FINP_TOK][MLAP_NOPE] = reinterpret_cast<uint16_t(*)[FINP_TOK][MLAP_NOPE]>(lds + FINP_WAVES * FIN_W_BYTES);
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int head = wg % p.n_heads;
+    const int nblocks = (p.T + FINP_TOK - 1) / FINP_TOK;
+    const int b0 = (wg / p.n_heads) * per;
+    const int b1 = b0 + per < nblocks ? b0 + per : nblocks;
+    const int ncols = p.n_heads * MLAP_QHEAD;
+    const int colbase = 64 * w;
+
+    {   // this wave's slice: rows of 128 bytes, pitch 1024 bytes: 8 lanes per row, 8 rows per request
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(p.w_uk) + ((size_t)head * MLAP_NOPE + (l >> 3)) * (MLAP_KV * 2) +
+                             colbase * 2 + 16 * (l & 7);
+        const uint32_t dst = (uint32_t)(uintptr_t)(lds_byte_t *)(wsl + w * FIN_W_BYTES);
+#pragma unroll 1
+        for (int i = 0; i < MLAP_NOPE / 8; ++i) dma16(src + (size_t)i * 8 * MLAP_KV * 2, dst + 1024 * i);
+    }
+    // lane l: nope channels 2l, 2l+1; lanes < 32: rope channels 2l, 2l+1 (= rotation partners l, 32+l)
+    auto load = [&](FinRaw &r, const int blk) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = blk * FINP_TOK + 4 * w + u;
+            const int tt = t < p.T ? t : p.T - 1;
+            const int32_t *row = p.qpart + (size_t)tt * ncols + head * MLAP_QHEAD;
+            r.ts[u] = p.q_norm_scale[tt];
+            r.nope[u] = *reinterpret_cast<const int2 *>(row + 2 * l);
+            if (l < 32) {
+                r.rope[u] = *reinterpret_cast<const int2 *>(row + MLAP_NOPE + 2 * l);
+                r.c0[u] = p.cos[(size_t)tt * MLAP_ROPE + l];
+                r.c1[u] = p.cos[(size_t)tt * MLAP_ROPE + 32 + l];
+                r.s0[u] = p.sin[(size_t)tt * MLAP_ROPE + l];
+                r.s1[u] = p.sin[(size_t)tt * MLAP_ROPE + 32 + l];
+            }
+        }
+    };
+    const f32x2 cs_nope = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + head * MLAP_QHEAD + 2 * l);
+    const f32x2 cs_rope = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + head * MLAP_QHEAD + MLAP_NOPE + 2 * (l & 31));
+    FinRaw raw;
+    if (b0 < b1) load(raw, b0);
+    VM_WAIT(0);
+
+    const uint16_t *wt = reinterpret_cast<const uint16_t *>(wsl + w * FIN_W_BYTES) +
+                         (4 * (l >> 5) + ((l & 15) >> 2)) * 64 + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+#pragma unroll 1
+    for (int blk = b0; blk < b1; ++blk) {
+        const int buf = (blk - b0) & 1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int tl = 4 * w + u;
+            const int t = blk * FINP_TOK + tl;
+            const float ts = raw.ts[u];
+            const float a0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.nope[u].x, ts), cs_nope[0]));
+            const float a1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.nope[u].y, ts), cs_nope[1]));
+            *reinterpret_cast<uint32_t *>(&abf[buf][tl][2 * l]) = pack_bf16x2(a0, a1);
+            if (l < 32 && t < p.T) {
+                const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.rope[u].x, ts), cs_rope[0]));
+                const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.rope[u].y, ts), cs_rope[1]));
+                const float r0 = __builtin_fmaf(v0, bf16_bits_to_f32(raw.c0[u]), (-v1) * bf16_bits_to_f32(raw.s0[u]));
+                const float r1 = __builtin_fmaf(v1, bf16_bits_to_f32(raw.c1[u]), v0 * bf16_bits_to_f32(raw.s1[u]));
+                uint16_t *out = p.q_rope + ((size_t)t * p.n_heads + head) * MLAP_ROPE;
+                out[l] = (uint16_t)(pack_bf16x2(r0, 0.f) & 0xffffu);
+                out[32 + l] = (uint16_t)(pack_bf16x2(r1, 0.f) & 0xffffu);
+            }
+        }
+        if (blk + 1 < b1) load(raw, blk + 1);
+        __syncthreads();                               // this block's operands are complete; the other buffer is free
+
+        const uint16_t *at = &abf[buf][l & 31][4 * (l >> 5)];
+        f32x16 c[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c[cb][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < MLAP_NOPE / 16; ++ks) {
+            const u32x2 bq0 = *reinterpret_cast<const u32x2 *>(at + 16 * ks);
+            const u32x2 bq1 = *reinterpret_cast<const u32x2 *>(at + 16 * ks + 8);
+            const u32x4 bq = {bq0[0], bq0[1], bq1[0], bq1[1]};
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb) {
+                const s16x4 a0 = lds_read_tr16(wt + (16 * ks) * 64 + 32 * cb);
+                const s16x4 a1 = lds_read_tr16(wt + (16 * ks + 8) * 64 + 32 * cb);
+                const s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+                c[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, bq), c[cb], 0, 0, 0);
+            }
+        }
+        const int t = blk * FINP_TOK + (l & 31);
+        if (t < p.T) {
+            uint16_t *dst = p.q_nope + ((size_t)t * p.n_heads + head) * MLAP_KV + colbase + 4 * (l >> 5);
+#pragma unroll
+            for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const u32x2 v = {pack_bf16x2(c[cb][4 * q], c[cb][4 * q + 1]), pack_bf16x2(c[cb][4 * q + 2], c[cb][4 * q + 3])};
+                    *reinterpret_cast<u32x2 *>(dst + 32 * cb + 8 * q) = v;
+                }
+        }
+    }
+}
 
 }  // namespace
 }  // namespace pto

@@ -37,6 +37,12 @@ hipError_t prolog_fused_launch(const MlapParams &pm, const LipParams &pl, hipStr
     if (e != hipSuccess) return e;
     e = lip_launch_linear(pl, stream);
     if (e != hipSuccess) return e;
+    if (mlap_finish_is_prefill(pm)) {
+        // prefill sizes: the attention query's last stage has a form of its own (one workgroup per compute unit)
+        e = mlap_launch_finish(pm, stream);
+        if (e != hipSuccess) return e;
+        return lip_launch_finish(pl, stream);
+    }
     const int mla_wgs = mlap_finish_wgs(pm);
     const int q_wgs = lip_finish_query_wgs(pl);
     hipLaunchKernelGGL(prolog_fused_finish_kernel, dim3((unsigned)(mla_wgs + q_wgs + pl.T)), dim3(64 * FIN_WAVES), 0, stream, pm, pl,

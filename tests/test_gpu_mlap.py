@@ -171,6 +171,63 @@ def test_mla_prolog_feeds_the_attention_cache_layout():
         assert np.abs(deq.reshape(512)).max() > 0
 
 
+def run_fused(dm, dl, t, n, n_idx, op=None):
+    """The fused operator on device inputs dm (MLA prolog) and dl (indexer prolog); caches updated in place."""
+    dev = dm.token_x.device
+    q_nope = torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev)
+    q_rope = torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev)
+    q_int8 = torch.empty([t, n_idx, 128], dtype=torch.int8, device=dev)
+    q_scale = torch.empty([t, n_idx, 1], dtype=torch.float16, device=dev)
+    weights = torch.empty([t, n_idx], dtype=torch.float16, device=dev)
+    ret = (op or pypto_amd.mla_indexer_prolog_quant_d)(
+        dm.token_x, dm.w_dq, dm.w_uq_qr, dm.dequant_scale, dm.w_uk, dm.w_dkv_kr, dm.gamma_cq, dm.gamma_ckv, dm.cos, dm.sin,
+        dm.cache_index, dm.kv_cache, dm.kr_cache, dm.k_scale_cache, dl.w_qb, dl.w_qb_scale, dl.wk, dl.w_proj, dl.ln_gamma_k,
+        dl.ln_beta_k, dl.hadamard_q, dl.hadamard_k, dl.k_cache, dl.k_cache_scale, q_nope, q_rope, dm.kv_cache, dm.kr_cache,
+        dm.k_scale_cache, q_int8, q_scale, dl.k_cache, dl.k_cache_scale, weights, 1e-5, 1e-5, "PA_BSND",
+        pypto_amd.MlaTileConfig(), pypto_amd.IndexerPrologQuantAttr(), pypto_amd.IndexerPrologQuantConfigs(),
+        pypto_amd.RopeTileShapeConfig())
+    assert ret is None
+    torch.cuda.synchronize()
+    return q_nope, q_rope, q_int8, q_scale, weights
+
+
+@pytest.mark.parametrize("exact", [False, True])
+def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(exact):
+    """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
+    projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
+    indexer prolog called one after the other on the same inputs, bit for bit, in both summation modes."""
+    from pypto_amd import mla_prolog_quant_impl as impl
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs
+    impl.EXACT_ABSORB = exact
+    kw = dict(h=256, q_lora_rank=512)
+    b, s1, act = 3, 50, [700, 650, 600]
+    dev = torch.device("cuda:0")
+    mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=4, **kw)
+    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=4, **kw)
+    t = b * s1
+    # separate operators
+    sep = run_op(mla, (1e-5, 1e-5), prefill=True)
+    dl = lip.to(dev)
+    la = list(dl.input_tensors())
+    dm0 = mla.to(dev)
+    la[0], la[1], la[2] = dm0.token_x, torch.from_numpy(sep["q_norm"]).to(dev), torch.from_numpy(sep["q_norm_scale"]).reshape(-1, 1).to(dev)
+    la[9], la[10], la[15] = dm0.cos, dm0.sin, dm0.cache_index
+    s_q = torch.empty([t, 4, 128], dtype=torch.int8, device=dev)
+    s_sc = torch.empty([t, 4, 1], dtype=torch.float16, device=dev)
+    s_w = torch.empty([t, 4], dtype=torch.float16, device=dev)
+    pypto_amd.lightning_indexer_prolog_quant(*la, s_q, s_sc, dl.k_cache, dl.k_cache_scale, s_w)
+    torch.cuda.synchronize()
+    # fused
+    dm, dl2 = mla.to(dev), lip.to(dev)
+    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl2, t, 4, 4, op=pypto_amd.mla_indexer_prolog_quant_p)
+    assert np.array_equal(q_nope.float().cpu().numpy(), sep["query_nope"])
+    assert np.array_equal(q_rope.float().cpu().numpy(), sep["query_rope"])
+    assert np.array_equal(dm.kv_cache.cpu().numpy(), sep["kv_cache"])
+    assert np.array_equal(dm.kr_cache.float().cpu().numpy(), sep["kr_cache"])
+    assert torch.equal(q_int8, s_q) and torch.equal(q_scale, s_sc) and torch.equal(weights, s_w)
+    assert torch.equal(dl2.k_cache, dl.k_cache) and torch.equal(dl2.k_cache_scale, dl.k_cache_scale)
+
+
 def test_fused_mla_indexer_prolog_matches_the_oracle_chain():
     """mla_indexer_prolog_quant_d: the indexer prolog consumes the MLA prolog's hidden q_norm / q_norm_scale; the
     ten outputs equal the two oracles chained (cos/sin of the MLA generator's range feed both stages)."""
@@ -188,21 +245,7 @@ def test_fused_mla_indexer_prolog_matches_the_oracle_chain():
 
     dev = torch.device("cuda:0")
     dm, dl = mla.to(dev), lip.to(dev)
-    t, n = 4, 4
-    q_nope = torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev)
-    q_rope = torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev)
-    q_int8 = torch.empty([t, n, 128], dtype=torch.int8, device=dev)
-    q_scale = torch.empty([t, n, 1], dtype=torch.float16, device=dev)
-    weights = torch.empty([t, n], dtype=torch.float16, device=dev)
-    ret = pypto_amd.mla_indexer_prolog_quant_d(
-        dm.token_x, dm.w_dq, dm.w_uq_qr, dm.dequant_scale, dm.w_uk, dm.w_dkv_kr, dm.gamma_cq, dm.gamma_ckv, dm.cos, dm.sin,
-        dm.cache_index, dm.kv_cache, dm.kr_cache, dm.k_scale_cache, dl.w_qb, dl.w_qb_scale, dl.wk, dl.w_proj, dl.ln_gamma_k,
-        dl.ln_beta_k, dl.hadamard_q, dl.hadamard_k, dl.k_cache, dl.k_cache_scale, q_nope, q_rope, dm.kv_cache, dm.kr_cache,
-        dm.k_scale_cache, q_int8, q_scale, dl.k_cache, dl.k_cache_scale, weights, 1e-5, 1e-5, "PA_BSND",
-        pypto_amd.MlaTileConfig(), pypto_amd.IndexerPrologQuantAttr(), pypto_amd.IndexerPrologQuantConfigs(),
-        pypto_amd.RopeTileShapeConfig())
-    assert ret is None
-    torch.cuda.synchronize()
+    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl, 4, 4, 4)
     assert np.array_equal(q_nope.float().cpu().numpy(), r_mla["query_nope"])
     assert np.array_equal(q_rope.float().cpu().numpy(), r_mla["query_rope"])
     assert np.array_equal(dm.kv_cache.cpu().numpy(), r_mla["kv_cache"])
