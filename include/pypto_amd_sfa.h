@@ -306,7 +306,18 @@ typedef struct PtoLiPrologQuantArgs {
     int64_t n_heads;
     int64_t cache_rows;   /* block_num * block_size */
     float eps;            /* layer-norm epsilon (attrs.eps) */
-    int32_t reserved;
+    int32_t sum_mode;     /* how the fp32 sums are taken from 64 tokens on (below that always in the fixed order
+                             above, bit-reproducible):
+                             0 (what a zero-initialised struct gives): the query rows' Hadamard sums on the matrix
+                               cores -- the same exact bf16 products added in the cores' order, so q_int8 may
+                               differ by one step and q_scale in its last bit in rare rows, which the reference's
+                               acceptance rule for these two outputs allows
+                               (deepseekv32_lightning_indexer_prolog_quant.py:424-425); the key row and the
+                               weights, for which that rule allows no outlier (:426-428), keep the fixed order;
+                             1: every sum in its fixed order;
+                             2: as 0, and the sums over h on the matrix cores as well (n_heads a multiple of 8): the
+                               fastest form; the key row's scale and the weights may then differ by one rounding
+                               step of their bf16 intermediate in rare entries. */
 } PtoLiPrologQuantArgs;
 
 int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *args, size_t *bytes);

@@ -316,9 +316,8 @@ int mlap_check(const PtoMlaPrologQuantArgs *a)
 // [group sums over the hidden axis | 4 partial int32 projections]
 size_t mlap_xpart_bytes(const PtoMlaPrologQuantArgs *a)
 {
-    const size_t nblk = (size_t)a->h / pto::MLAP_XBLOCK;
-    const size_t ngroups = (nblk + pto::MLAP_XGROUP - 1) / pto::MLAP_XGROUP;
-    const size_t bytes = ngroups * a->t * (a->q_lora_rank + pto::MLAP_KV + pto::MLAP_ROPE) * sizeof(float);
+    const size_t rows = (size_t)pto::mlap_xpart_rows((int)a->h, (int)a->t);
+    const size_t bytes = rows * a->t * (a->q_lora_rank + pto::MLAP_KV + pto::MLAP_ROPE) * sizeof(float);
     return (bytes + 255) & ~(size_t)255;
 }
 size_t mlap_ws_bytes(const PtoMlaPrologQuantArgs *a)
@@ -512,6 +511,7 @@ int pto_li_prolog_quant_workspace_bytes(const PtoLiPrologQuantArgs *a, size_t *b
 // checked arguments -> kernel parameters
 static int lip_params(const PtoLiPrologQuantArgs *a, pto::LipParams &p)
 {
+    if (a && (a->sum_mode < 0 || a->sum_mode > 2)) return fail(PTO_E_INVALID_ARG, "li_prolog: sum_mode must be 0, 1 or 2");
     int rc = lip_check(a);
     if (rc != PTO_OK) return rc;
     if (!a->x || !a->q_norm || !a->q_norm_scale || !a->w_qb || !a->w_qb_scale || !a->wk || !a->w_proj || !a->ln_gamma_k ||
@@ -555,6 +555,7 @@ static int lip_params(const PtoLiPrologQuantArgs *a, pto::LipParams &p)
     p.q_lora = (int)a->q_lora_rank;
     p.n_heads = (int)a->n_heads;
     p.eps = a->eps;
+    p.sum_mode = a->sum_mode;
     p.w_mul0 = (float)std::pow((double)a->n_heads, -0.5);
     p.w_mul1 = (float)std::pow((double)pto::LIP_DIM, -0.5);
     return PTO_OK;

@@ -40,7 +40,36 @@ struct LipParams {
     long long cache_rows;
     int T, h, q_lora, n_heads;
     float eps, w_mul0, w_mul1;   // weights = fp16((bf16(x.w_proj) * w_mul0) * w_mul1)
+    int sum_mode;                // LIP_SUMS_*
 };
+
+// How the fp32 sums are taken from LIP_MFMA_MIN_TOKENS tokens on (below that every sum has its fixed order):
+constexpr int LIP_SUMS_DEFAULT = 0;        // the query rows' Hadamard sums on the matrix cores, everything else fixed-order
+constexpr int LIP_SUMS_EXACT = 1;          // every sum in its fixed order
+constexpr int LIP_SUMS_MATRIX_CORES = 2;   // the sums over the hidden axis on the matrix cores as well
+constexpr int LIP_MFMA_MIN_TOKENS = 64;
+constexpr int LIP_XM_MAX_SPLITS = 16;    // ranges of the hidden axis (partial sums per token) of the matrix-core form, at most
+
+__host__ __device__ inline bool lip_q_on_matrix_cores(const LipParams &p)
+{
+    return p.T >= LIP_MFMA_MIN_TOKENS && p.sum_mode != LIP_SUMS_EXACT;
+}
+// the hidden-axis form needs w_proj rows made of whole 16-byte pieces
+__host__ __device__ inline bool lip_x_on_matrix_cores(const LipParams &p)
+{
+    return p.T >= LIP_MFMA_MIN_TOKENS && p.sum_mode == LIP_SUMS_MATRIX_CORES && p.n_heads % 8 == 0;
+}
+// partial rows [T, LIP_XCOLS] the first launch leaves per token: the blocks of 64 of the fixed-order form, or the
+// ranges of the matrix-core form (enough of them for about 256 workgroups of 128 tokens x 128 columns)
+__host__ __device__ inline int lip_xrows(const LipParams &p)
+{
+    const int nblk = p.h / LIP_XBLOCK;
+    if (!lip_x_on_matrix_cores(p)) return nblk;
+    int s = 128 / ((p.T + 127) / 128);
+    s = s < 1 ? 1 : s;
+    s = s > LIP_XM_MAX_SPLITS ? LIP_XM_MAX_SPLITS : s;
+    return s > nblk ? nblk : s;
+}
 
 hipError_t lip_launch(const LipParams &p, hipStream_t stream);
 // the first launch alone, and the number of query-row workgroups of the second (for the fused operator's last launch)

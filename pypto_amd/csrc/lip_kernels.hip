@@ -32,6 +32,7 @@
 #include "lip_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"
+#include "xlinear_mfma.h"
 
 #pragma clang fp contract(off)
 
@@ -170,6 +171,31 @@ __global__ __launch_bounds__(256) void lip_qproj_prefill_kernel(const QProj p, c
     q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
+// The sums over the hidden axis on the matrix cores (xlinear_mfma.h): workgroup = (wk or w_proj, one of nsplit
+// ranges of the hidden axis, 128 tokens); w_proj is a narrow slab of n_heads columns.
+static_assert(XM_KC == LIP_XBLOCK, "the workspace is sized in chunks of the hidden axis");
+__global__ __launch_bounds__(256) void lip_xlinear_mfma_kernel(const LipParams p, const int nsplit)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XM_LDS];
+    const int slab = blockIdx.x & 1;
+    const int sp = (blockIdx.x >> 1) % nsplit;
+    const int t0 = ((blockIdx.x >> 1) / nsplit) * XM_TOK;
+    XmSlab sl;
+    sl.w = reinterpret_cast<const uint8_t *>(slab ? p.w_proj : p.wk);
+    sl.pitch = (slab ? p.n_heads : LIP_DIM) * 2;
+    sl.pieces = slab ? p.n_heads / 8 : 16;
+    sl.out = p.xpart + (size_t)sp * p.T * LIP_XCOLS + slab * LIP_DIM;
+    sl.out_pitch = LIP_XCOLS;
+    const int nchunks = p.h / XM_KC;
+    xm_body(sl, p.x, p.T, p.h, t0, (int)((long long)sp * nchunks / nsplit), (int)((long long)(sp + 1) * nchunks / nsplit), smem);
+}
+
+__global__ __launch_bounds__(64 * QFP_WAVES) void lip_finish_query_prefill_kernel(const LipParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LIP_QFP_LDS];
+    lip_finish_query_prefill_body(p, (int)blockIdx.x, (int)gridDim.x, lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second launch: prolog_finish.h.
 __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
@@ -180,7 +206,8 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipPar
 
 }  // namespace
 
-int lip_finish_query_wgs(const LipParams &p) { return (p.T * p.n_heads + FIN_WAVES - 1) / FIN_WAVES; }
+// workgroups of the second launch that finish query rows (none where the rows have a launch of their own)
+int lip_finish_query_wgs(const LipParams &p) { return lip_q_on_matrix_cores(p) ? 0 : (p.T * p.n_heads + FIN_WAVES - 1) / FIN_WAVES; }
 
 hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
 {
@@ -195,6 +222,12 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
         hipLaunchKernelGGL(lip_qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+    }
+    if (lip_x_on_matrix_cores(p)) {
+        const int nsplit = lip_xrows(p);
+        const int ttiles = (p.T + XM_TOK - 1) / XM_TOK;
+        hipLaunchKernelGGL(lip_xlinear_mfma_kernel, dim3((unsigned)(2 * nsplit * ttiles)), dim3(256), 0, stream, p, nsplit);
+        return hipGetLastError();
     }
     const int x_jobs = 2 * (p.h / LIP_XBLOCK) * ((p.T + XTOK - 1) / XTOK);
     // enough workgroups that each hidden-axis wave gets about one job, never fewer than the query jobs
@@ -221,6 +254,17 @@ hipError_t lip_launch(const LipParams &p, hipStream_t stream)
 hipError_t lip_launch_finish(const LipParams &p, hipStream_t stream)
 {
     const int q_wgs = lip_finish_query_wgs(p);
+    if (lip_q_on_matrix_cores(p)) {
+        // the query rows on the matrix cores, in passes of 32 rows per wave, at most two workgroups per compute unit
+        const int npass = (p.T * p.n_heads + 31) / 32;
+        const int cus = cu_count();
+        if (cus <= 0) return hipErrorNoDevice;
+        int wgs = (npass + QFP_WAVES - 1) / QFP_WAVES;
+        wgs = wgs > 2 * cus ? 2 * cus : wgs;
+        hipLaunchKernelGGL(lip_finish_query_prefill_kernel, dim3((unsigned)wgs), dim3(64 * QFP_WAVES), 0, stream, p);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     hipLaunchKernelGGL(lip_finish_kernel, dim3((unsigned)(q_wgs + p.T)), dim3(64 * FIN_WAVES), 0, stream, p, q_wgs);
     return hipGetLastError();
 }

@@ -16,6 +16,17 @@ constexpr int MLAP_MAX_QLORA = 1536;
 constexpr int QPROJ_KSPLIT_HOST = 4; // partial sums of the int8 projection (prolog_common.h: QPROJ_KSPLIT)
 constexpr int MLAP_XTOK = 8;         // tokens per job of the first and of the last kernel
 constexpr int MLAP_MFMA_MIN_TOKENS = 64;   // from here on the first launch sums on the matrix cores (unless absorb_exact)
+constexpr int MLAP_XM_MAX_SPLITS = 8;      // ranges of the hidden axis (partial sums per token) of that form, at most
+
+// rows [T, q_lora + 576] of partial sums over the hidden axis the workspace holds: the group sums of the
+// fixed-order form, or the ranges of the matrix-core form where that may run
+inline int mlap_xpart_rows(const int h, const int T)
+{
+    const int nblk = h / MLAP_XBLOCK;
+    const int groups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
+    const int splits = T >= MLAP_MFMA_MIN_TOKENS ? (nblk < MLAP_XM_MAX_SPLITS ? nblk : MLAP_XM_MAX_SPLITS) : 0;
+    return groups > splits ? groups : splits;
+}
 
 struct MlapParams {
     const uint16_t *x;            // [T, h] bf16

@@ -30,6 +30,7 @@
 #include "mlap_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"
+#include "xlinear_mfma.h"
 
 #pragma clang fp contract(off)
 
@@ -134,144 +135,28 @@ __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapP
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill form of the first launch: the same product on the matrix cores, for 64 tokens and more when the caller
-// has not asked for the fixed-order sums.  All products are exact in fp32 as before; the sums over the hidden
-// axis are taken in the cores' own order, so the results may differ from the fixed-order ones in the last bit
-// (and the int8 latents that follow, rarely, by one step).
-//   workgroup = (slab of 128 columns, quarter of the hidden axis or less, 128 tokens), four waves: wave (wc, wt)
-//   holds columns 64*wc .. +63 x tokens 64*wt .. +63 as four 32x32 accumulators of
-//   O^T[column][token] = sum_k W^T[column][k] x^T[k][token]
-//   A = W^T: the slab's rows are row-major [k][128 columns], so the operand is read from LDS with the
-//   transposing ds_read_b64_tr_b16; B = x^T: lane (token, half) holds 8 consecutive hidden states of its token.
-//   Chunks of 64 hidden rows travel by LDS-DMA into two buffers (16 KiB of the slab + 16 KiB of hidden states
-//   each), the next chunk under the products of the current one.  16-byte piece q of slab row r sits at piece
-//   q ^ 4*(r & 3), piece q of token row t at q ^ ((t >> 1) & 7): the four rows of a transposing read and the 32
-//   token rows of an operand read then spread over all banks.
-constexpr int XM_TOK = 128;                      // tokens per workgroup
-constexpr int XM_KC = 64;                        // hidden rows per chunk
-constexpr int XM_W_BYTES = XM_KC * 256;          // slab rows are staged 256 bytes apart (a half slab fills half)
-constexpr int XM_X_BYTES = XM_TOK * XM_KC * 2;
-constexpr int XM_BUF = XM_W_BYTES + XM_X_BYTES;
-constexpr int XM_MAX_SPLITS = 4;
+// Prefill form of the first launch: the same product on the matrix cores (xlinear_mfma.h), for 64 tokens and more
+// when the caller has not asked for the fixed-order sums.  workgroup = (slab of 128 columns of [w_dq | w_dkv_kr],
+// one of nsplit ranges of the hidden axis, 128 tokens); the 64 rope columns are a narrow slab of their own.
+static_assert(XM_KC == MLAP_XBLOCK, "the workspace is sized in chunks of the hidden axis");
 
 __global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams p, const int nslabs, const int nsplit)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * XM_BUF];
-    const int l = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wc = w & 1, wt = w >> 1;
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XM_LDS];
     const int slab = blockIdx.x % nslabs;
     const int sp = (blockIdx.x / nslabs) % nsplit;
     const int t0 = (blockIdx.x / nslabs / nsplit) * XM_TOK;
     const int qslabs = p.q_lora / 128;
     const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
     const bool isq = slab < qslabs;
-    const uint8_t *wbase = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256
-                               : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
-    const int pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
-    const bool half_slab = !isq && slab - qslabs == 4;             // the 64 rope columns
+    XmSlab sl;
+    sl.w = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256 : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
+    sl.pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
+    sl.pieces = !isq && slab - qslabs == 4 ? 8 : 16;
+    sl.out = p.xpart + (size_t)sp * p.T * nc + slab * 128;
+    sl.out_pitch = nc;
     const int nchunks = p.h / XM_KC;
-    const int c_begin = (int)((long long)sp * nchunks / nsplit);
-    const int c_end = (int)((long long)(sp + 1) * nchunks / nsplit);
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_byte_t *)smem;
-
-    // this wave's eight requests of a chunk: four of the slab (four rows each), four of the hidden states (eight
-    // token rows each)
-    const int wrow = l >> 4, wpos = l & 15;
-    const uint32_t woff = (uint32_t)(wrow * pitch + 16 * (half_slab ? wpos : (wpos ^ (4 * wrow))));
-    const uint64_t wmask = half_slab ? 0x00FF00FF00FF00FFull : ~0ull;
-    const int xrow = l >> 3, xpos = l & 7;
-    auto request_chunk = [&](const int c, const int buf) {
-        const uint32_t dst = lds0 + (uint32_t)(buf * XM_BUF);
-        const uint8_t *wsrc = wbase + (size_t)(c * XM_KC) * pitch + woff;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int req = 4 * w + j;
-            dma16_lanes(wsrc + (size_t)(4 * req) * pitch, dst + 1024u * req, wmask);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int req = 4 * w + j;
-            const int tl = 8 * req + xrow;                          // token row inside the workgroup's 128
-            int t = t0 + tl;
-            t = t < p.T ? t : p.T - 1;
-            dma16(reinterpret_cast<const uint8_t *>(p.x) + ((size_t)t * p.h + (size_t)c * XM_KC) * 2 + 16 * (xpos ^ ((tl >> 1) & 7)),
-                  dst + XM_W_BYTES + 1024u * req);
-        }
-    };
-
-    f32x16 acc[2][2];
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[cb][tb][r] = 0.f;
-
-    // per-lane read offsets inside a buffer
-    // A: row 16*ks + 8*(l>>5) + (l&15)>>2 (+4), column 64*wc + 32*cb + 16*((l>>4)&1) + 4*(l&3)
-    const int arow = 8 * (l >> 5) + ((l & 15) >> 2);
-    const int aswz = half_slab ? 0 : 4 * ((l & 15) >> 2);
-    uint32_t aoff[2];
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-        const int piece = 8 * wc + 4 * cb + 2 * ((l >> 4) & 1) + ((l & 3) >> 1);
-        aoff[cb] = (uint32_t)(arow * 256 + 16 * (piece ^ aswz) + 8 * (l & 1));
-    }
-    // B: token row 64*wt + 32*tb + (l&31), piece 2*ks + (l>>5)
-    const int brow = 64 * wt + (l & 31);
-    const int bswz = (brow >> 1) & 7;
-    if (c_begin < c_end) request_chunk(c_begin, 0);
-    for (int c = c_begin; c < c_end; ++c) {
-        const int buf = (c - c_begin) & 1;
-        if (c + 1 < c_end) {
-            request_chunk(c + 1, buf ^ 1);
-            VM_WAIT(8);
-        } else {
-            VM_WAIT(0);
-        }
-        __syncthreads();                                           // every wave's part of the chunk has landed
-        const uint8_t *wb = smem + buf * XM_BUF;
-        const uint8_t *xb = wb + XM_W_BYTES;
-        if (!(half_slab && wc == 1)) {
-#pragma unroll
-            for (int ks = 0; ks < XM_KC / 16; ++ks) {
-                bf16x8 a[2], b[2];
-#pragma unroll
-                for (int cb = 0; cb < 2; ++cb) {
-                    const uint16_t *ap = reinterpret_cast<const uint16_t *>(wb + aoff[cb] + 16 * ks * 256);
-                    const s16x4 lo = lds_read_tr16(ap), hi = lds_read_tr16(ap + 4 * 128);
-                    a[cb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                }
-#pragma unroll
-                for (int tb = 0; tb < 2; ++tb)
-                    b[tb] = *reinterpret_cast<const bf16x8 *>(xb + (brow + 32 * tb) * 128 + 16 * ((2 * ks + (l >> 5)) ^ bswz));
-#pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-                    for (int tb = 0; tb < 2; ++tb)
-                        acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cb], b[tb], acc[cb][tb], 0, 0, 0);
-            }
-        }
-        __syncthreads();                                           // the buffer may be requested into again
-    }
-    // accumulator register r of lane (token, half) is column 8*(r/4) + 4*half + r%4 of its 32-column block
-    if (!(half_slab && wc == 1)) {
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
-            const int t = t0 + 64 * wt + 32 * tb + (l & 31);
-            if (t < p.T) {
-                float *dst = p.xpart + ((size_t)sp * p.T + t) * nc + slab * 128 + 64 * wc + 4 * (l >> 5);
-#pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const f32x4 v = {acc[cb][tb][4 * q], acc[cb][tb][4 * q + 1], acc[cb][tb][4 * q + 2], acc[cb][tb][4 * q + 3]};
-                        *reinterpret_cast<f32x4 *>(dst + 32 * cb + 8 * q) = v;
-                    }
-            }
-        }
-    }
+    xm_body(sl, p.x, p.T, p.h, t0, (int)((long long)sp * nchunks / nsplit), (int)((long long)(sp + 1) * nchunks / nsplit), smem);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -476,9 +361,15 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
     const int nslabs = p.q_lora / 128 + 5;
     if (p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact) {
         // prefill sizes: the sums over the hidden axis on the matrix cores, up to four partial sums per token
+        // as many ranges as give about two workgroups per compute unit (one is resident at a time, by its LDS)
         const int nchunks = p.h / XM_KC;
-        ngroups = nchunks < XM_MAX_SPLITS ? nchunks : XM_MAX_SPLITS;
         const int ttiles = (p.T + XM_TOK - 1) / XM_TOK;
+        const int cus = cu_count();
+        if (cus <= 0) return hipErrorNoDevice;
+        ngroups = 2 * cus / (nslabs * ttiles);
+        ngroups = ngroups < 1 ? 1 : ngroups;
+        ngroups = ngroups > MLAP_XM_MAX_SPLITS ? MLAP_XM_MAX_SPLITS : ngroups;
+        ngroups = ngroups > nchunks ? nchunks : ngroups;
         hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)(nslabs * ngroups * ttiles)), dim3(256), 0, stream, p, nslabs, ngroups);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;

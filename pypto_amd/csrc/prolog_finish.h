@@ -164,7 +164,7 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
     }
 
     const int t = wg - q_wgs;
-    const int nblk = p.h / LIP_XBLOCK;
+    const int nblk = lip_xrows(p);
     const int ngroups = (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
     stage_matrix(hmat, p.hk);
     const bool pl = l < p.n_heads;
@@ -242,6 +242,125 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
     }
 }
 
+
+// The query rows at prefill sizes with the Hadamard sums on the matrix cores: a workgroup of four waves stages the
+// matrix once (rows padded to 272 bytes so that the four rows of a transposing read fall into different banks),
+// then each wave walks passes of 32 rows (token, head): it de-quantises and rotates its rows, eight at a time, into
+// its own bf16 operand buffer, takes O^T[j][row] = sum_i H^T[j][i] a^T[i][row] as 32 products
+// (v_mfma_f32_32x32x16_bf16, A = the matrix read transposed, B = the rows), rounds to bf16, quantises each row
+// (lanes l and l + 32 hold one row between them) and sends the int8 rows through its buffer so that they leave as
+// whole 16-byte pieces.  All products are exact; the sums run in the cores' order instead of i ascending.
+constexpr int QFP_WAVES = 4;
+constexpr int QFP_HPITCH = 136;                        // elements between matrix rows in LDS
+constexpr int QFP_APITCH = 136;                        // elements between operand rows
+constexpr int QFP_OPITCH = 144;                        // bytes between int8 rows on their way out
+constexpr int QFP_WAVE_BYTES = 32 * QFP_APITCH * 2;
+constexpr int LIP_QFP_LDS = LIP_DIM * QFP_HPITCH * 2 + QFP_WAVES * QFP_WAVE_BYTES;   // 69 632 bytes
+static_assert(32 * QFP_OPITCH <= QFP_WAVE_BYTES, "the int8 rows reuse the operand buffer");
+
+__device__ __forceinline__ void lip_finish_query_prefill_body(const LipParams &p, const int wg, const int nwg, uint8_t *lds)
+{
+    uint16_t *hmat = reinterpret_cast<uint16_t *>(lds);
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint8_t *mine = lds + LIP_DIM * QFP_HPITCH * 2 + w * QFP_WAVE_BYTES;
+    uint16_t *abf = reinterpret_cast<uint16_t *>(mine);
+    {
+        const u32x4 *s = reinterpret_cast<const u32x4 *>(p.hq);
+        for (int i = threadIdx.x; i < LIP_DIM * LIP_DIM / 8; i += 64 * QFP_WAVES)
+            *reinterpret_cast<u32x4 *>(hmat + (i >> 4) * QFP_HPITCH + (i & 15) * 8) = s[i];
+    }
+    __syncthreads();
+    const int ncols = p.n_heads * LIP_DIM;
+    const int nrows = p.T * p.n_heads;
+    const int npass = (nrows + 31) / 32;
+    const uint16_t *at = abf + (l & 31) * QFP_APITCH + 4 * (l >> 5);
+    const uint16_t *wt = hmat + (4 * (l >> 5) + ((l & 15) >> 2)) * QFP_HPITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
+#pragma unroll 1
+    for (int pass = wg * QFP_WAVES + w; pass < npass; pass += nwg * QFP_WAVES) {
+#pragma unroll 1
+        for (int b8 = 0; b8 < 4; ++b8) {
+            int2 raw[8];
+            float ts[8];
+            f32x2 cs[8];
+            uint32_t rc[8], rs[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int row = pass * 32 + b8 * 8 + u;
+                const int rr = row < nrows ? row : nrows - 1;
+                const int t = rr / p.n_heads;
+                const int col = (rr - t * p.n_heads) * LIP_DIM + 2 * l;
+                raw[u] = *reinterpret_cast<const int2 *>(p.qpart + (size_t)t * ncols + col);
+                ts[u] = p.q_norm_scale[t];
+                cs[u] = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
+                rc[u] = rope_coef(p.cos, t, l);
+                rs[u] = rope_coef(p.sin, t, l);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw[u].x, ts[u]), cs[u][0]));
+                float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw[u].y, ts[u]), cs[u][1]));
+                rope_pair(v0, v1, rc[u], rs[u], l);
+                *reinterpret_cast<uint32_t *>(abf + (b8 * 8 + u) * QFP_APITCH + 2 * l) = pack_bf16x2(v0, v1);
+            }
+        }
+        // the wave reads back what it wrote itself: LDS operations of a wave stay in order
+        f32x16 c[4];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) c[cb][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < LIP_DIM / 16; ++ks) {
+            const u32x2 b0 = *reinterpret_cast<const u32x2 *>(at + 16 * ks);
+            const u32x2 b1 = *reinterpret_cast<const u32x2 *>(at + 16 * ks + 8);
+            const u32x4 bq = {b0[0], b0[1], b1[0], b1[1]};
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb) {
+                const s16x4 a0 = lds_read_tr16(wt + (16 * ks) * QFP_HPITCH + 32 * cb);
+                const s16x4 a1 = lds_read_tr16(wt + (16 * ks + 8) * QFP_HPITCH + 32 * cb);
+                const s16x8 a = __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7);
+                c[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, bq), c[cb], 0, 0, 0);
+            }
+        }
+        // lane (row, half) holds channels 32*cb + 8*(r/4) + 4*half + r%4 of its row
+        float amax = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                c[cb][r] = bf16_round_f32(c[cb][r]);
+                amax = fmaxf(amax, fabsf(c[cb][r]));
+            }
+        {
+            const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(amax), __float_as_uint(amax), false, false);
+            amax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+        }
+        float s = 0.f, deq = 0.f;
+        if (amax > 0.f) {
+            s = __fdiv_rn(127.0f, amax);
+            deq = __fdiv_rn(1.0f, s);
+        }
+        uint8_t *orow = mine + (l & 31) * QFP_OPITCH + 4 * (l >> 5);
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint32_t v = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v |= (uint32_t)((int)rintf(__fmul_rn(c[cb][4 * g + j], s)) & 0xff) << (8 * j);
+                *reinterpret_cast<uint32_t *>(orow + 32 * cb + 8 * g) = v;
+            }
+        const int row = pass * 32 + (l & 31);
+        if (l < 32 && row < nrows) p.q_scale[row] = (uint16_t)(pack_f16x2(deq, 0.f) & 0xffffu);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int r = 8 * k + (l >> 3);
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(mine + r * QFP_OPITCH + 16 * (l & 7));
+            if (pass * 32 + r < nrows) *reinterpret_cast<u32x4 *>(p.q_int8 + (size_t)(pass * 32 + r) * LIP_DIM + 16 * (l & 7)) = v;
+        }
+    }
+}
 
 // ---------------------------------------------------------------------------------- MLA prolog
 constexpr int FIN_W_BYTES = MLAP_NOPE * 64 * 2;    // a wave's slice of w_uk[head]: 128 rows x 64 columns bf16
@@ -398,7 +517,8 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
 // per 8 tokens; each output has the bits of the decode form (same products, same order).
 constexpr int FINP_TOK = 32;
 constexpr int FINP_WAVES = 8;
-constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * MLAP_NOPE * 2;   // 147 456 bytes
+constexpr int FINP_APITCH = MLAP_NOPE + 8;   // elements between operand rows: 272 bytes, so that the 32 rows of an operand read spread over the banks
+constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_APITCH * 2;   // 148 480 bytes
 static_assert(MLAP_MFMA_MIN_TOKENS >= QPROJ_PREFILL_TOKENS, "the prefill form reads one partial sum per output");
 
 struct FinRaw {
@@ -410,7 +530,7 @@ struct FinRaw {
 __device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, const int wg, const int per, uint8_t *lds)
 {
     uint8_t *wsl = lds;
-    uint16_t(*abf)[FINP_TOK][MLAP_NOPE] = reinterpret_cast<uint16_t(*)[FINP_TOK][MLAP_NOPE]>(lds + FINP_WAVES * FIN_W_BYTES);
+    uint16_t(*abf)[FINP_TOK][FINP_APITCH] = reinterpret_cast<uint16_t(*)[FINP_TOK][FINP_APITCH]>(lds + FINP_WAVES * FIN_W_BYTES);
     const int l = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int head = wg % p.n_heads;

@@ -37,8 +37,8 @@ hipError_t prolog_fused_launch(const MlapParams &pm, const LipParams &pl, hipStr
     if (e != hipSuccess) return e;
     e = lip_launch_linear(pl, stream);
     if (e != hipSuccess) return e;
-    if (mlap_finish_is_prefill(pm)) {
-        // prefill sizes: the attention query's last stage has a form of its own (one workgroup per compute unit)
+    if (mlap_finish_is_prefill(pm) || lip_q_on_matrix_cores(pl)) {
+        // prefill sizes: the last stages have forms of their own (the attention query's: one workgroup per compute unit)
         e = mlap_launch_finish(pm, stream);
         if (e != hipSuccess) return e;
         return lip_launch_finish(pl, stream);

@@ -208,8 +208,9 @@ PYBIND11_MODULE(_C, m)
              std::uintptr_t cos_idx_rope, std::uintptr_t sin_idx_rope, std::uintptr_t hadamard_q, std::uintptr_t hadamard_k,
              std::uintptr_t k_cache, std::uintptr_t k_cache_scale, std::uintptr_t k_cache_index, std::uintptr_t q_int8,
              std::uintptr_t q_scale, std::uintptr_t weights, std::uintptr_t workspace, size_t workspace_bytes, int64_t t,
-             int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows, double eps, std::uintptr_t stream) {
+             int64_t h, int64_t q_lora_rank, int64_t n_heads, int64_t cache_rows, double eps, int sum_mode, std::uintptr_t stream) {
               PtoLiPrologQuantArgs a{};
+              a.sum_mode = sum_mode;
               a.x = ptr<const void>(x);
               a.q_norm = ptr<const int8_t>(q_norm);
               a.q_norm_scale = ptr<const float>(q_norm_scale);
@@ -297,7 +298,7 @@ PYBIND11_MODULE(_C, m)
     auto fused_args = [](const std::vector<std::uintptr_t> &m, const std::vector<std::uintptr_t> &x, std::uintptr_t workspace,
                          size_t workspace_bytes, int64_t t, int64_t h, int64_t q_lora_rank, int64_t mla_heads,
                          int64_t mla_cache_rows, double epsilon_cq, double epsilon_ckv, bool absorb_exact, int64_t idx_heads,
-                         int64_t idx_cache_rows, double idx_eps) {
+                         int64_t idx_cache_rows, double idx_eps, int idx_sum_mode) {
         if (m.size() != 18 || x.size() != 19) throw std::invalid_argument("mla_indexer_prolog: 18 + 19 pointers expected");
         PtoMlaIndexerPrologQuantArgs a{};
         a.mla.token_x = ptr<const void>(m[0]);
@@ -342,6 +343,7 @@ PYBIND11_MODULE(_C, m)
         a.indexer.n_heads = idx_heads;
         a.indexer.cache_rows = idx_cache_rows;
         a.indexer.eps = static_cast<float>(idx_eps);
+        a.indexer.sum_mode = idx_sum_mode;
         a.workspace = ptr<void>(workspace);
         a.workspace_bytes = workspace_bytes;
         return a;
@@ -351,7 +353,7 @@ PYBIND11_MODULE(_C, m)
                        int64_t idx_cache_rows) {
               const std::vector<std::uintptr_t> m18(18, 0), x19(19, 0);
               PtoMlaIndexerPrologQuantArgs a = fused_args(m18, x19, 0, 0, t, h, q_lora_rank, mla_heads, mla_cache_rows, 0.0, 0.0,
-                                                          false, idx_heads, idx_cache_rows, 0.0);
+                                                          false, idx_heads, idx_cache_rows, 0.0, 0);
               size_t bytes = 0;
               check(pto_mla_indexer_prolog_quant_workspace_bytes(&a, &bytes));
               return bytes;
@@ -360,10 +362,10 @@ PYBIND11_MODULE(_C, m)
           [fused_args](const std::vector<std::uintptr_t> &mla_ptrs, const std::vector<std::uintptr_t> &idx_ptrs,
                        std::uintptr_t workspace, size_t workspace_bytes, int64_t t, int64_t h, int64_t q_lora_rank,
                        int64_t mla_heads, int64_t mla_cache_rows, double epsilon_cq, double epsilon_ckv, bool absorb_exact,
-                       int64_t idx_heads, int64_t idx_cache_rows, double idx_eps, std::uintptr_t stream) {
+                       int64_t idx_heads, int64_t idx_cache_rows, double idx_eps, int idx_sum_mode, std::uintptr_t stream) {
               PtoMlaIndexerPrologQuantArgs a = fused_args(mla_ptrs, idx_ptrs, workspace, workspace_bytes, t, h, q_lora_rank,
                                                           mla_heads, mla_cache_rows, epsilon_cq, epsilon_ckv, absorb_exact,
-                                                          idx_heads, idx_cache_rows, idx_eps);
+                                                          idx_heads, idx_cache_rows, idx_eps, idx_sum_mode);
               check(pto_mla_indexer_prolog_quant_launch(&a, ptr<void>(stream)));
           });
 }

@@ -1,0 +1,157 @@
+// Sums over the hidden axis on the matrix cores, for prefill-sized token counts: x [T, h] bf16 times a slab of up
+// to 128 columns of a row-major bf16 weight matrix, as partial sums over a range of the hidden axis.  Shared by the
+// MLA prolog (w_dq, w_dkv_kr) and the lightning-indexer prolog (wk, w_proj); included after prolog_common.h.
+//
+// All products are exact in fp32 (bf16 x bf16); the sums are taken in the cores' own order, so the results may
+// differ from the fixed-order sums of the decode kernels in the last bit.
+//   workgroup = (slab, range of the hidden axis, 128 tokens), four waves: wave (wc, wt) holds columns
+//   64*wc .. +63 x tokens 64*wt .. +63 as four 32x32 accumulators of
+//   O^T[column][token] = sum_k W^T[column][k] x^T[k][token]
+//   A = W^T: the slab's rows are row-major [k][columns], so the operand is read from LDS with the transposing
+//   ds_read_b64_tr_b16; B = x^T: lane (token, half) holds 8 consecutive hidden states of its token.
+//   Chunks of 64 hidden rows travel by LDS-DMA into XM_NBUF buffers (16 KiB of the slab + 16 KiB of hidden states
+//   each), XM_NBUF - 1 chunks ahead of the products.  16-byte piece q of slab row r sits at piece q ^ 4*(r & 3),
+//   piece q of token row t at q ^ ((t >> 1) & 7): the four rows of a transposing read and the 32 token rows of an
+//   operand read then spread over all banks.  A slab narrower than 128 columns (8 * pieces) is staged unswizzled
+//   by the lanes whose pieces exist; the columns past its end hold whatever the buffer held and are not stored.
+#pragma once
+#include "prolog_common.h"
+
+namespace pto {
+namespace {
+
+constexpr int XM_TOK = 128;                      // tokens per workgroup
+constexpr int XM_KC = 64;                        // hidden rows per chunk
+constexpr int XM_W_BYTES = XM_KC * 256;          // slab rows are staged 256 bytes apart
+constexpr int XM_X_BYTES = XM_TOK * XM_KC * 2;
+constexpr int XM_BUF = XM_W_BYTES + XM_X_BYTES;
+constexpr int XM_NBUF = 3;
+constexpr int XM_LDS = XM_NBUF * XM_BUF;
+
+struct XmSlab {
+    const uint8_t *w;     // column 0 of the slab in row 0 of the weight matrix
+    int pitch;            // bytes between rows of the weight matrix
+    int pieces;           // 16-byte pieces of a row that belong to the slab: 16, or fewer for a narrow one
+    float *out;           // partial sums of this range: out[t * out_pitch + column of the slab]
+    int out_pitch;
+};
+
+// chunks [c_begin, c_end) of the hidden axis, tokens t0 .. t0 + 127 (rows past T - 1 repeat it and are not stored)
+__device__ __forceinline__ void xm_body(const XmSlab &sl, const uint16_t *x, const int T, const int h, const int t0, const int c_begin,
+                                        const int c_end, uint8_t *smem)
+{
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wc = w & 1, wt = w >> 1;
+    const bool narrow = sl.pieces < 16;
+    const bool idle = sl.pieces <= 8 && wc == 1;                   // no column of this wave's half exists
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_byte_t *)smem;
+
+    // this wave's eight requests of a chunk: four of the slab (four rows each), four of the hidden states (eight
+    // token rows each)
+    const int wrow = l >> 4, wpos = l & 15;
+    const uint32_t woff = (uint32_t)(wrow * sl.pitch + 16 * (narrow ? (wpos < sl.pieces ? wpos : 0) : (wpos ^ (4 * wrow))));
+    const uint64_t wmask = narrow ? ((1ull << sl.pieces) - 1) * 0x0001000100010001ull : ~0ull;
+    const int xrow = l >> 3, xpos = l & 7;
+    auto request_chunk = [&](const int c, const int buf) {
+        const uint32_t dst = lds0 + (uint32_t)(buf * XM_BUF);
+        const uint8_t *wsrc = sl.w + (size_t)(c * XM_KC) * sl.pitch + woff;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int req = 4 * w + j;
+            dma16_lanes(wsrc + (size_t)(4 * req) * sl.pitch, dst + 1024u * req, wmask);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int req = 4 * w + j;
+            const int tl = 8 * req + xrow;                          // token row inside the workgroup's 128
+            int t = t0 + tl;
+            t = t < T ? t : T - 1;
+            dma16(reinterpret_cast<const uint8_t *>(x) + ((size_t)t * h + (size_t)c * XM_KC) * 2 + 16 * (xpos ^ ((tl >> 1) & 7)),
+                  dst + XM_W_BYTES + 1024u * req);
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[cb][tb][r] = 0.f;
+
+    // per-lane read offsets inside a buffer
+    // A: row 16*ks + 8*(l>>5) + (l&15)>>2 (+4), column 64*wc + 32*cb + 16*((l>>4)&1) + 4*(l&3)
+    const int arow = 8 * (l >> 5) + ((l & 15) >> 2);
+    const int aswz = narrow ? 0 : 4 * ((l & 15) >> 2);
+    uint32_t aoff[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+        const int piece = 8 * wc + 4 * cb + 2 * ((l >> 4) & 1) + ((l & 3) >> 1);
+        aoff[cb] = (uint32_t)(arow * 256 + 16 * (piece ^ aswz) + 8 * (l & 1));
+    }
+    // B: token row 64*wt + 32*tb + (l&31), piece 2*ks + (l>>5)
+    const int brow = 64 * wt + (l & 31);
+    const int bswz = (brow >> 1) & 7;
+    // XM_NBUF - 1 chunks are on their way while one is multiplied; a chunk is eight requests per wave
+#pragma unroll
+    for (int i = 0; i < XM_NBUF - 1; ++i)
+        if (c_begin + i < c_end) request_chunk(c_begin + i, i);
+    int buf = 0;
+#pragma unroll 1
+    for (int c = c_begin; c < c_end; ++c) {
+        const int ahead = c_end - 1 - c;                           // chunks requested after this one
+        if (ahead >= XM_NBUF - 2) VM_WAIT(8 * (XM_NBUF - 2));
+        else if (XM_NBUF > 3 && ahead == 1) VM_WAIT(8);
+        else VM_WAIT(0);
+        __syncthreads();                                           // every wave's part of chunk c has landed, and
+                                                                   // every wave is done with chunk c - 1
+        if (c + XM_NBUF - 1 < c_end) request_chunk(c + XM_NBUF - 1, buf == 0 ? XM_NBUF - 1 : buf - 1);
+        const uint8_t *wb = smem + buf * XM_BUF;
+        const uint8_t *xb = wb + XM_W_BYTES;
+        if (!idle) {
+#pragma unroll
+            for (int ks = 0; ks < XM_KC / 16; ++ks) {
+                bf16x8 a[2], b[2];
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb) {
+                    const uint16_t *ap = reinterpret_cast<const uint16_t *>(wb + aoff[cb] + 16 * ks * 256);
+                    const s16x4 lo = lds_read_tr16(ap), hi = lds_read_tr16(ap + 4 * 128);
+                    a[cb] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb)
+                    b[tb] = *reinterpret_cast<const bf16x8 *>(xb + (brow + 32 * tb) * 128 + 16 * ((2 * ks + (l >> 5)) ^ bswz));
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int tb = 0; tb < 2; ++tb)
+                        acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cb], b[tb], acc[cb][tb], 0, 0, 0);
+            }
+        }
+        buf = buf + 1 == XM_NBUF ? 0 : buf + 1;
+    }
+    // accumulator register r of lane (token, half) is column 8*(r/4) + 4*half + r%4 of its 32-column block
+    if (!idle) {
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) {
+            const int t = t0 + 64 * wt + 32 * tb + (l & 31);
+            if (t < T) {
+                const int col0 = 64 * wc + 4 * (l >> 5);
+                float *dst = sl.out + (size_t)t * sl.out_pitch + col0;
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (col0 + 32 * cb + 8 * q < 8 * sl.pieces) {
+                            const f32x4 v = {acc[cb][tb][4 * q], acc[cb][tb][4 * q + 1], acc[cb][tb][4 * q + 2], acc[cb][tb][4 * q + 3]};
+                            *reinterpret_cast<f32x4 *>(dst + 32 * cb + 8 * q) = v;
+                        }
+                    }
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace pto

@@ -15,6 +15,16 @@ Outputs are pre-allocated by the caller and written in place: ``q_int8_out``, ``
 (``k_int8_out``/``k_scale_out`` normally alias ``k_int8_in``/``k_scale_in``, as in the reference driver
 :404-405; when they do not, the cache is copied first).  Returns ``None``; runs asynchronously on the
 current stream.
+
+Every fp32 sum has a fixed order and the results are bit-reproducible below 64 tokens.  From 64 tokens on (prefill
+chunks) two module attributes choose: by default the query rows' Hadamard sums run on the matrix cores -- the same
+exact products added in the cores' order; ``q_int8`` may then differ by one step and ``q_scale`` in its last bit in
+rare rows, which the reference's acceptance rule allows for these outputs
+(deepseekv32_lightning_indexer_prolog_quant.py:424-425) -- while the key row and the weights, for which that rule
+allows no outlier, keep their fixed order.  ``EXACT_SUMS = True`` keeps every sum in its fixed order at any size;
+``MATRIX_CORE_HIDDEN_SUMS = True`` also takes the sums over the hidden axis on the matrix cores (``n_heads`` a multiple
+of 8), the fastest form: the key row's scale and the weights may then differ by one rounding step of their bf16
+intermediate in rare entries.
 """
 from __future__ import annotations
 
@@ -80,6 +90,12 @@ class IndexerPrologQuantConfigs:
 
 
 HEAD_DIM = 128
+EXACT_SUMS = False
+MATRIX_CORE_HIDDEN_SUMS = False
+
+
+def _sum_mode() -> int:
+    return 1 if EXACT_SUMS else (2 if MATRIX_CORE_HIDDEN_SUMS else 0)
 ROPE_DIM = 64
 
 
@@ -158,7 +174,7 @@ def lightning_indexer_prolog_quant(x_in, q_norm_in, q_norm_scale_in, w_qb_in, w_
         # half of the fused operator: checked here, launched by the caller together with the other half
         _collect.append(dict(ptrs=[v.data_ptr() for v in (x, qn, qns, wqb, wqbs, wk, wp, gam, bet, cos, sin, hq, hk, kc, ks, kidx,
                                                           qo, qso, wo)],
-                             t=t, h=h, q_lora=q_lora, n_heads=n_heads, cache_rows=cache_rows, eps=float(attrs.eps)))
+                             t=t, h=h, q_lora=q_lora, n_heads=n_heads, cache_rows=cache_rows, eps=float(attrs.eps), sum_mode=_sum_mode()))
         return None
     ws_bytes = C.li_prolog_quant_workspace_bytes(t, h, q_lora, n_heads, cache_rows)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -168,5 +184,5 @@ def lightning_indexer_prolog_quant(x_in, q_norm_in, q_norm_scale_in, w_qb_in, w_
                                  wk.data_ptr(), wp.data_ptr(), gam.data_ptr(), bet.data_ptr(), cos.data_ptr(),
                                  sin.data_ptr(), hq.data_ptr(), hk.data_ptr(), kc.data_ptr(), ks.data_ptr(),
                                  kidx.data_ptr(), qo.data_ptr(), qso.data_ptr(), wo.data_ptr(), ws.data_ptr(), ws_bytes,
-                                 t, h, q_lora, n_heads, cache_rows, float(attrs.eps), stream)
+                                 t, h, q_lora, n_heads, cache_rows, float(attrs.eps), _sum_mode(), stream)
     return None

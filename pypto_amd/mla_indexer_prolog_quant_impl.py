@@ -63,7 +63,7 @@ def _fused(mla_op, token_x, mla_w_dq, mla_w_uq_qr, mla_dequant_scale, mla_w_uk, 
     with torch.cuda.device(x.device):
         C.mla_indexer_prolog_quant_launch(m["ptrs"], i["ptrs"], ws.data_ptr(), ws_bytes, m["t"], m["h"], m["q_lora"],
                                           m["n_heads"], m["cache_rows"], m["eps_cq"], m["eps_ckv"], m["absorb_exact"],
-                                          i["n_heads"], i["cache_rows"], i["eps"], stream)
+                                          i["n_heads"], i["cache_rows"], i["eps"], i["sum_mode"], stream)
     return None
 
 

@@ -12,6 +12,17 @@ from pypto_amd.synthetic import gen_indexer_prolog_inputs
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def exact_sums():
+    """The bit-exact tests below run every sum in its fixed order at any size; the matrix-core forms the operator takes
+    by default from 64 tokens on are tested against the reference's acceptance rule at the end of the file."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as impl
+    old = impl.EXACT_SUMS
+    impl.EXACT_SUMS = True
+    yield
+    impl.EXACT_SUMS = old
+
+
 def run_op(inp, separate_cache_out=False):
     dev = torch.device("cuda:0")
     d = inp.to(dev)
@@ -111,3 +122,72 @@ def test_prolog_reference_large_cases(b, s1, act, what):
     inp = gen_indexer_prolog_inputs(b, s1, act, seed=b + s1)
     ref = lo.indexer_prolog_ref(*inp.input_tensors())
     assert_exact(run_op(inp), ref, what)
+
+
+PREFILL_CASES = [
+    (3, 50, [700, 650, 600], dict(h=256, q_lora_rank=512, n_heads=8)),     # 150 tokens: ragged token tiles, one piece of w_proj per row
+    (1, 77, [300], dict(h=192, q_lora_rank=1024, n_heads=24)),             # three chunks of the hidden axis, ragged row passes
+    (32, 4, [2048 + 17 * i for i in range(32)], {}),                       # 128 tokens at the model's sizes
+    (128, 4, [8192] * 128, {}),                                            # 512 tokens
+    (1, 4096, [65536], {}),                                                # 4096 tokens of one sequence
+]
+
+
+def untouched_rows_equal(got, ref, rows):
+    mask = np.ones(got["k_cache"].reshape(-1, 128).shape[0], dtype=bool)
+    mask[rows] = False
+    return np.array_equal(got["k_cache"].reshape(-1, 128)[mask], ref["k_cache"].reshape(-1, 128)[mask])
+
+
+@pytest.mark.parametrize("b,s1,act,kw", PREFILL_CASES + [(2, 40, [500, 400], dict(h=128, q_lora_rank=512, n_heads=3))])
+def test_prolog_prefill_sizes_default_sums(b, s1, act, kw):
+    """The operator's default from 64 tokens on: the query rows' Hadamard sums on the matrix cores (same exact
+    products, the cores' summation order), everything else in its fixed order.  Key rows, key scales and weights --
+    for which the reference's acceptance rule allows no outlier (deepseekv32_lightning_indexer_prolog_quant.py:426-428)
+    -- equal the sequential statement bit for bit; q_int8 within one step and q_scale within 2.5e-5 but for at most
+    0.5 % of the rows, as that rule allows (:424-425)."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as impl
+    impl.EXACT_SUMS = False
+    inp = gen_indexer_prolog_inputs(b, s1, act, seed=b + s1 + 1, **kw)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    got = run_op(inp)
+    for name in ("k_cache", "k_cache_scale", "weights"):
+        assert np.array_equal(got[name].view(np.uint8 if got[name].dtype == np.int8 else np.uint16),
+                              ref[name].view(np.uint8 if ref[name].dtype == np.int8 else np.uint16)), name
+    dq = np.abs(got["q_int8"].astype(np.int32) - ref["q_int8"].astype(np.int32))
+    assert dq.max() <= 1
+    ds = np.abs(got["q_scale"].astype(np.float32) - ref["q_scale"].astype(np.float32))
+    assert (ds > 2.5e-5).mean() <= 0.005
+    print(f"t={b * s1}: q_int8 off by one {float((dq != 0).mean()):.6f}, q_scale differs in {float((ds != 0).mean()):.6f} of the rows "
+          f"(max {float(ds.max()):.2e})", flush=True)
+
+
+@pytest.mark.parametrize("b,s1,act,kw", PREFILL_CASES)
+def test_prolog_prefill_sizes_hidden_sums_on_matrix_cores(b, s1, act, kw):
+    """MATRIX_CORE_HIDDEN_SUMS: the sums over the hidden axis on the matrix cores as well.  int8 rows within one
+    step; key scales and weights within 2.5e-5 of the sequential statement but for rare entries (at most 0.5 %) where
+    the bf16 value they are made from rounds the other way -- never more than that one step (2^-7 relative)."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as impl
+    impl.EXACT_SUMS = False
+    impl.MATRIX_CORE_HIDDEN_SUMS = True
+    try:
+        inp = gen_indexer_prolog_inputs(b, s1, act, seed=b + s1 + 1, **kw)
+        ref = lo.indexer_prolog_ref(*inp.input_tensors())
+        got = run_op(inp)
+    finally:
+        impl.MATRIX_CORE_HIDDEN_SUMS = False
+    rows = inp.k_cache_index.numpy()
+    dq = np.abs(got["q_int8"].astype(np.int32) - ref["q_int8"].astype(np.int32))
+    assert dq.max() <= 1
+    ds = np.abs(got["q_scale"].astype(np.float32) - ref["q_scale"].astype(np.float32))
+    assert (ds > 2.5e-5).mean() <= 0.005
+    gk, rk = got["k_cache"].reshape(-1, 128)[rows].astype(np.int32), ref["k_cache"].reshape(-1, 128)[rows].astype(np.int32)
+    assert np.abs(gk - rk).max() <= 1
+    gs, rs = got["k_cache_scale"].reshape(-1)[rows].astype(np.float32), ref["k_cache_scale"].reshape(-1)[rows].astype(np.float32)
+    assert (np.abs(gs - rs) > 2.5e-5).mean() <= 0.005 and np.all(np.abs(gs - rs) <= 2.5e-5 + 0.0078125 * np.abs(rs))
+    gw, rw = got["weights"].astype(np.float32), ref["weights"].astype(np.float32)
+    assert (np.abs(gw - rw) > 2.5e-5).mean() <= 0.005 and np.all(np.abs(gw - rw) <= 2.5e-5 + 0.0078125 * np.abs(rw))
+    assert untouched_rows_equal(got, ref, rows)
+    print(f"t={b * s1}: q_int8 off by one {float((dq != 0).mean()):.6f}, key entries off by one {float((gk != rk).mean()):.6f}, "
+          f"key scales beyond 2.5e-5: {int((np.abs(gs - rs) > 2.5e-5).sum())} of {gs.size}, "
+          f"weights beyond 2.5e-5: {int((np.abs(gw - rw) > 2.5e-5).sum())} of {gw.size}", flush=True)

@@ -14,13 +14,15 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True)
 def exact_absorb():
-    """The bit-exact comparisons below want the fixed-order form of the product with w_uk; the matrix-core form
-    (the operator's default) has a test of its own."""
+    """The bit-exact tests run both prologs with every sum in its fixed order; the matrix-core forms have tests of
+    their own that switch them on."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd import mla_prolog_quant_impl as impl
-    old = impl.EXACT_ABSORB
+    old = impl.EXACT_ABSORB, lip_impl.EXACT_SUMS, lip_impl.MATRIX_CORE_HIDDEN_SUMS
     impl.EXACT_ABSORB = True
+    lip_impl.EXACT_SUMS = True
     yield
-    impl.EXACT_ABSORB = old
+    impl.EXACT_ABSORB, lip_impl.EXACT_SUMS, lip_impl.MATRIX_CORE_HIDDEN_SUMS = old
 
 
 def run_op(inp, eps=(0.0, 0.0), separate_cache_out=False, prefill=False):
@@ -191,19 +193,21 @@ def run_fused(dm, dl, t, n, n_idx, op=None):
     return q_nope, q_rope, q_int8, q_scale, weights
 
 
-@pytest.mark.parametrize("exact", [False, True])
-def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(exact):
+@pytest.mark.parametrize("mode", ["default", "exact", "matrix_cores"])
+def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode):
     """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
     projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
-    indexer prolog called one after the other on the same inputs, bit for bit, in both summation modes."""
+    indexer prolog called one after the other on the same inputs, bit for bit, in each of the summation modes."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd import mla_prolog_quant_impl as impl
     from pypto_amd.synthetic import gen_indexer_prolog_inputs
-    impl.EXACT_ABSORB = exact
+    impl.EXACT_ABSORB = lip_impl.EXACT_SUMS = mode == "exact"
+    lip_impl.MATRIX_CORE_HIDDEN_SUMS = mode == "matrix_cores"
     kw = dict(h=256, q_lora_rank=512)
     b, s1, act = 3, 50, [700, 650, 600]
     dev = torch.device("cuda:0")
     mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=4, **kw)
-    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=4, **kw)
+    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=8, **kw)
     t = b * s1
     # separate operators
     sep = run_op(mla, (1e-5, 1e-5), prefill=True)
@@ -212,14 +216,14 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(exact):
     dm0 = mla.to(dev)
     la[0], la[1], la[2] = dm0.token_x, torch.from_numpy(sep["q_norm"]).to(dev), torch.from_numpy(sep["q_norm_scale"]).reshape(-1, 1).to(dev)
     la[9], la[10], la[15] = dm0.cos, dm0.sin, dm0.cache_index
-    s_q = torch.empty([t, 4, 128], dtype=torch.int8, device=dev)
-    s_sc = torch.empty([t, 4, 1], dtype=torch.float16, device=dev)
-    s_w = torch.empty([t, 4], dtype=torch.float16, device=dev)
+    s_q = torch.empty([t, 8, 128], dtype=torch.int8, device=dev)
+    s_sc = torch.empty([t, 8, 1], dtype=torch.float16, device=dev)
+    s_w = torch.empty([t, 8], dtype=torch.float16, device=dev)
     pypto_amd.lightning_indexer_prolog_quant(*la, s_q, s_sc, dl.k_cache, dl.k_cache_scale, s_w)
     torch.cuda.synchronize()
     # fused
     dm, dl2 = mla.to(dev), lip.to(dev)
-    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl2, t, 4, 4, op=pypto_amd.mla_indexer_prolog_quant_p)
+    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl2, t, 4, 8, op=pypto_amd.mla_indexer_prolog_quant_p)
     assert np.array_equal(q_nope.float().cpu().numpy(), sep["query_nope"])
     assert np.array_equal(q_rope.float().cpu().numpy(), sep["query_rope"])
     assert np.array_equal(dm.kv_cache.cpu().numpy(), sep["kv_cache"])
@@ -278,7 +282,7 @@ def test_fused_entry_point_through_the_c_abi_keeps_the_intermediates_in_its_work
                                       "cos_idx_rope", "sin_idx_rope", "hadamard_q", "hadamard_k", "k_cache", "k_cache_scale",
                                       "k_cache_index", "q_int8", "q_scale", "weights", "workspace")] + \
                    [("workspace_bytes", ctypes.c_size_t)] + [(n, i64) for n in ("t", "h", "q_lora_rank", "n_heads", "cache_rows")] + \
-                   [("eps", f32), ("reserved", i32)]
+                   [("eps", f32), ("sum_mode", i32)]
 
     class Fused(ctypes.Structure):
         _fields_ = [("mla", Mla), ("indexer", Idx), ("workspace", vp), ("workspace_bytes", ctypes.c_size_t)]
