@@ -59,11 +59,19 @@ __host__ __device__ inline bool lip_x_on_matrix_cores(const LipParams &p)
 {
     return p.T >= LIP_MFMA_MIN_TOKENS && p.sum_mode == LIP_SUMS_MATRIX_CORES && p.n_heads % 8 == 0;
 }
+// the fixed-order sums over the hidden axis at prefill sizes leave one row per group of eight blocks (the group sums)
+// instead of one per block; the staging of that form needs w_proj rows of a power of two of 16-byte pieces
+__host__ __device__ inline bool lip_x_group_rows(const LipParams &p)
+{
+    const int wb = p.n_heads * 2;
+    return p.T >= LIP_MFMA_MIN_TOKENS && !lip_x_on_matrix_cores(p) && wb >= 16 && (wb & (wb - 1)) == 0;
+}
 // partial rows [T, LIP_XCOLS] the first launch leaves per token: the blocks of 64 of the fixed-order form, or the
 // ranges of the matrix-core form (enough of them for about 256 workgroups of 128 tokens x 128 columns)
 __host__ __device__ inline int lip_xrows(const LipParams &p)
 {
     const int nblk = p.h / LIP_XBLOCK;
+    if (lip_x_group_rows(p)) return (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
     if (!lip_x_on_matrix_cores(p)) return nblk;
     int s = 128 / ((p.T + 127) / 128);
     s = s < 1 ? 1 : s;

@@ -30,6 +30,7 @@
 #include "mlap_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"
+#include "xlinear_fixed.h"
 #include "xlinear_mfma.h"
 
 #pragma clang fp contract(off)
@@ -39,99 +40,26 @@ namespace {
 
 static_assert(QPROJ_KSPLIT == QPROJ_KSPLIT_HOST, "workspace sizing and kernels disagree");
 
-constexpr int XL_WAVES = MLAP_XGROUP;                                  // one block per wave
-constexpr int XL_W_BYTES = MLAP_XBLOCK * 256;                          // a block of one slab: 64 rows x 256 bytes
-constexpr int XL_REGION = XL_W_BYTES + MLAP_XTOK * MLAP_XBLOCK * 4;    // + the hidden states as fp32
+static_assert(XL_BLOCK == MLAP_XBLOCK && XL_GROUP == MLAP_XGROUP && XL_TOK == MLAP_XTOK, "workspace sizing and kernels disagree");
 
-// Column slabs: 0 .. q_lora/128 - 1 of w_dq, then four slabs of w_dkv_kr's latent part and one half slab
-// (64 columns) of its rope part.
+// Fixed-order sums over the hidden axis (xlinear_fixed.h).  Column slabs: 0 .. q_lora/128 - 1 of w_dq, then four
+// slabs of w_dkv_kr's latent part and one half slab (64 columns) of its rope part.
 __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapParams p, const int nslabs, const int ngroups)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[XL_WAVES * XL_REGION];
-    const int l = threadIdx.x & 63;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XL_LDS];
     const int slab = blockIdx.x % nslabs;
     const int g = (blockIdx.x / nslabs) % ngroups;
-    const int t0 = (blockIdx.x / nslabs / ngroups) * MLAP_XTOK;
+    const int t0 = (blockIdx.x / nslabs / ngroups) * XL_TOK;
     const int qslabs = p.q_lora / 128;
-    const int nblk = p.h / MLAP_XBLOCK;
     const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
-    // the slab's matrix, row pitch and width in bytes
     const bool isq = slab < qslabs;
-    const uint8_t *wbase = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256
-                               : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
-    const int pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
-    const int wbytes = (!isq && slab - qslabs == 4) ? 128 : 256;
-
-    uint8_t *region = smem + w * XL_REGION;
-    float *xs = reinterpret_cast<float *>(region + XL_W_BYTES);         // [8][64]
-    const int c = g * MLAP_XGROUP + w;                                    // this wave's block
-    const int nb = nblk - g * MLAP_XGROUP < MLAP_XGROUP ? nblk - g * MLAP_XGROUP : MLAP_XGROUP;
-    float a0[MLAP_XTOK], a1[MLAP_XTOK];
-#pragma unroll
-    for (int t = 0; t < MLAP_XTOK; ++t) a0[t] = a1[t] = 0.f;
-
-    if (w < nb) {
-        const int k0 = c * MLAP_XBLOCK;
-        const uint32_t wdst = (uint32_t)(uintptr_t)(lds_byte_t *)region;
-        {   // rows of wbytes bytes: wbytes/16 lanes per row
-            const int lpr = wbytes >> 4;
-            const int rpi = 64 / lpr;                                     // rows per request
-            const uint8_t *src = wbase + (size_t)(k0 + l / lpr) * pitch + 16 * (l % lpr);
-#pragma unroll 1
-            for (int i = 0; i < MLAP_XBLOCK / rpi; ++i) dma16(src + (size_t)i * rpi * pitch, wdst + 1024 * i);
-        }
-#pragma unroll
-        for (int u = 0; u < MLAP_XTOK / 2; ++u) {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + 2u + l/32
-            const int t = t0 + 2 * u + (l >> 5);
-            const int tt = t < p.T ? t : p.T - 1;
-            const uint32_t xv = reinterpret_cast<const uint32_t *>(p.x + (size_t)tt * p.h + k0)[l & 31];
-            f32x2 v = {__uint_as_float(xv << 16), __uint_as_float(xv & 0xffff0000u)};
-            *reinterpret_cast<f32x2 *>(xs + (2 * u + (l >> 5)) * MLAP_XBLOCK + 2 * (l & 31)) = v;
-        }
-        VM_WAIT(0);
-        const uint32_t *wl = reinterpret_cast<const uint32_t *>(region) + (wbytes == 256 ? l : (l & 31));
-        const int rowdw = wbytes >> 2;
-#pragma unroll 2
-        for (int kk = 0; kk < MLAP_XBLOCK; kk += 4) {
-            f32x4 xv[MLAP_XTOK];
-#pragma unroll
-            for (int t = 0; t < MLAP_XTOK; ++t) xv[t] = *reinterpret_cast<const f32x4 *>(xs + t * MLAP_XBLOCK + kk);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t wv = wl[(kk + j) * rowdw];
-                const float w0 = __uint_as_float(wv << 16), w1 = __uint_as_float(wv & 0xffff0000u);
-#pragma unroll
-                for (int t = 0; t < MLAP_XTOK; ++t) {
-                    a0[t] = __builtin_fmaf(xv[t][j], w0, a0[t]);
-                    a1[t] = __builtin_fmaf(xv[t][j], w1, a1[t]);
-                }
-            }
-        }
-        // block sums into this wave's own (consumed) region: [8 tokens][128 columns]
-        float *bs = reinterpret_cast<float *>(region);
-#pragma unroll
-        for (int t = 0; t < MLAP_XTOK; ++t) {
-            f32x2 v = {a0[t], a1[t]};
-            *reinterpret_cast<f32x2 *>(bs + t * 128 + 2 * l) = v;
-        }
-    }
-    __syncthreads();
-    // group sum: thread (token = w, columns 2l, 2l+1) chains the block sums in ascending order
-    {
-        const int t = t0 + w;
-        const int width = wbytes >> 1;                                    // columns of the slab
-        if (t < p.T && 2 * l < width) {
-            float s0 = 0.f, s1 = 0.f;
-            for (int i = 0; i < nb; ++i) {
-                const f32x2 v = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(smem + i * XL_REGION) + w * 128 + 2 * l);
-                s0 = __fadd_rn(s0, v[0]);
-                s1 = __fadd_rn(s1, v[1]);
-            }
-            f32x2 v = {s0, s1};
-            *reinterpret_cast<f32x2 *>(p.xpart + ((size_t)g * p.T + t) * nc + slab * 128 + 2 * l) = v;
-        }
-    }
+    XlSlab sl;
+    sl.w = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256 : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
+    sl.pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
+    sl.wbytes = (!isq && slab - qslabs == 4) ? 128 : 256;
+    sl.out = p.xpart + (size_t)g * p.T * nc + slab * 128;
+    sl.out_pitch = nc;
+    xl_body(sl, p.x, p.T, p.h, g, t0, smem);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -164,8 +164,9 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
     }
 
     const int t = wg - q_wgs;
-    const int nblk = lip_xrows(p);
-    const int ngroups = (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
+    const bool group_rows = lip_x_group_rows(p);       // the rows are group sums already
+    const int nblk = group_rows ? 0 : lip_xrows(p);
+    const int ngroups = group_rows ? lip_xrows(p) : (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
     stage_matrix(hmat, p.hk);
     const bool pl = l < p.n_heads;
     // everything wave 0 needs later is requested now
@@ -173,7 +174,14 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
     const uint32_t gm = reinterpret_cast<const uint32_t *>(p.gamma)[l];
     const uint32_t bt = reinterpret_cast<const uint32_t *>(p.beta)[l];
     const long long dst = p.k_cache_index[t];
-    for (int g0 = w; g0 < ngroups; g0 += 2 * FIN_WAVES) {
+    if (group_rows) {
+        for (int g = w; g < ngroups; g += FIN_WAVES) {
+            const float *r = p.xpart + ((size_t)g * p.T + t) * LIP_XCOLS;
+            *reinterpret_cast<f32x2 *>(&gsum[g][2 * l]) = *reinterpret_cast<const f32x2 *>(r + 2 * l);
+            gsum[g][LIP_DIM + l] = r[LIP_DIM + (pl ? l : 0)];
+        }
+    }
+    for (int g0 = w; g0 < ngroups && !group_rows; g0 += 2 * FIN_WAVES) {
         f32x2 kv[2][LIP_XGROUP];
         float wv[2][LIP_XGROUP];
         int nb[2];
