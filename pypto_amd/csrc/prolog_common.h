@@ -90,21 +90,32 @@ __device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const i
 #pragma unroll 1
         for (int s = 0; s < HS; ++s) dma16(src + 32 * s, tok + 1024 * s);
     }
-    {
+    {   // rows 16..31 of every step are staged with neighbours swapped (q_step_at)
         const int8_t *src = p.w + ((size_t)k0 + (l >> 3)) * ncols + head * 128 + 16 * (l & 7);
-#pragma unroll 2
-        for (int i = 0; i < NW; ++i) dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
+        const int8_t *swp = p.w + ((size_t)k0 + ((l >> 3) ^ 1)) * ncols + head * 128 + 16 * (l & 7);
+#pragma unroll 1
+        for (int i = 0; i < NW; i += 4) {
+            dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
+            dma16(src + (size_t)(i + 1) * 8 * ncols, tile + 1024 * (i + 1));
+            dma16(swp + (size_t)(i + 2) * 8 * ncols, tile + 1024 * (i + 2));
+            dma16(swp + (size_t)(i + 3) * 8 * ncols, tile + 1024 * (i + 3));
+        }
     }
 }
 
-// one 32-row step of the product: rows 32s.. of the tile, token operands of step s at tok + 1024 s
+// one 32-row step of the product: rows 32s.. of the tile, token operands of step s at tok + 1024 s.  Lanes 0..31
+// read rows 0..15 of the step, lanes 32..63 rows 16..31; a row is 32 dwords, so rows of the same parity share their
+// banks: rows 16..31 sit in LDS with neighbours swapped (row 16 + r at 16 + (r ^ 1)), which puts the two half-waves
+// of a read on opposite halves of the banks.
 __device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *tok, const int s, const int l, i32x16 (&acc)[4])
 {
     const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(tile);
-    const int rd = (16 * (l >> 5)) * 32 + (l & 31);     // dword index of this lane's first row of a step
+    const int hi = l >> 5;
+    const int rd = (16 * hi) * 32 + (l & 31);           // dword index of this lane's first row of a step
+    const int rd_even = rd + 32 * hi, rd_odd = rd - 32 * hi;
     uint32_t d[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + rd + r * 32];
+    for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + ((r & 1) ? rd_odd : rd_even) + r * 32];
     const i32x4 b = *reinterpret_cast<const i32x4 *>(tok + 1024 * s + 16 * l);
     i32x4 a[4];
 #pragma unroll
@@ -212,13 +223,14 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
     const int nch = p.q_lora / (32 * QPF_STEPS);
     const int8_t *tsrc = p.q_norm + (size_t)(t < p.T ? t : p.T - 1) * p.q_lora + 16 * (l >> 5);
     const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * (l & 7);
+    const int8_t *wswp = p.w + (size_t)(32 * w + ((l >> 3) ^ 1)) * ncols + slab * 128 + 16 * (l & 7);   // rows 16..31 of a step: neighbours swapped
     const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
     auto issue = [&](const int c) {
         const uint32_t buf = base + (c & 1) * QPF_BUF;
 #pragma unroll
         for (int s = 0; s < QPF_STEPS; ++s) dma16(tsrc + c * (32 * QPF_STEPS) + 32 * s, buf + QPF_TILE + w * QPF_TOK + 1024 * s);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(wsrc + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
+        for (int i = 0; i < 4; ++i) dma16((i < 2 ? wsrc : wswp) + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
     };
     i32x16 acc[4];
 #pragma unroll

@@ -9,8 +9,8 @@
 //   O^T[column][token] = sum_k W^T[column][k] x^T[k][token]
 //   A = W^T: the slab's rows are row-major [k][columns], so the operand is read from LDS with the transposing
 //   ds_read_b64_tr_b16; B = x^T: lane (token, half) holds 8 consecutive hidden states of its token.
-//   Chunks of 64 hidden rows travel by LDS-DMA into XM_NBUF buffers (16 KiB of the slab + 16 KiB of hidden states
-//   each), XM_NBUF - 1 chunks ahead of the products.  16-byte piece q of slab row r sits at piece q ^ 4*(r & 3),
+//   Chunks of 64 hidden rows travel by LDS-DMA into two buffers (16 KiB of the slab + 16 KiB of hidden states
+//   each), the next chunk under the products of the current one.  16-byte piece q of slab row r sits at piece q ^ 4*(r & 3),
 //   piece q of token row t at q ^ ((t >> 1) & 7): the four rows of a transposing read and the 32 token rows of an
 //   operand read then spread over all banks.  A slab narrower than 128 columns (8 * pieces) is staged unswizzled
 //   by the lanes whose pieces exist; the columns past its end hold whatever the buffer held and are not stored.
@@ -25,8 +25,7 @@ constexpr int XM_KC = 64;                        // hidden rows per chunk
 constexpr int XM_W_BYTES = XM_KC * 256;          // slab rows are staged 256 bytes apart
 constexpr int XM_X_BYTES = XM_TOK * XM_KC * 2;
 constexpr int XM_BUF = XM_W_BYTES + XM_X_BYTES;
-constexpr int XM_NBUF = 3;
-constexpr int XM_LDS = XM_NBUF * XM_BUF;
+constexpr int XM_LDS = 2 * XM_BUF;
 
 struct XmSlab {
     const uint8_t *w;     // column 0 of the slab in row 0 of the weight matrix
@@ -93,20 +92,19 @@ __device__ __forceinline__ void xm_body(const XmSlab &sl, const uint16_t *x, con
     // B: token row 64*wt + 32*tb + (l&31), piece 2*ks + (l>>5)
     const int brow = 64 * wt + (l & 31);
     const int bswz = (brow >> 1) & 7;
-    // XM_NBUF - 1 chunks are on their way while one is multiplied; a chunk is eight requests per wave
-#pragma unroll
-    for (int i = 0; i < XM_NBUF - 1; ++i)
-        if (c_begin + i < c_end) request_chunk(c_begin + i, i);
+    // the next chunk is requested into the other buffer before the current one is waited for; two workgroups share a
+    // compute unit, so eight waves keep requests in flight (the rate of LDS-DMA grows with the waves that issue it)
+    if (c_begin < c_end) request_chunk(c_begin, 0);
     int buf = 0;
 #pragma unroll 1
     for (int c = c_begin; c < c_end; ++c) {
-        const int ahead = c_end - 1 - c;                           // chunks requested after this one
-        if (ahead >= XM_NBUF - 2) VM_WAIT(8 * (XM_NBUF - 2));
-        else if (XM_NBUF > 3 && ahead == 1) VM_WAIT(8);
-        else VM_WAIT(0);
-        __syncthreads();                                           // every wave's part of chunk c has landed, and
-                                                                   // every wave is done with chunk c - 1
-        if (c + XM_NBUF - 1 < c_end) request_chunk(c + XM_NBUF - 1, buf == 0 ? XM_NBUF - 1 : buf - 1);
+        if (c + 1 < c_end) {
+            request_chunk(c + 1, buf ^ 1);
+            VM_WAIT(8);
+        } else {
+            VM_WAIT(0);
+        }
+        __syncthreads();                                           // every wave's part of chunk c has landed
         const uint8_t *wb = smem + buf * XM_BUF;
         const uint8_t *xb = wb + XM_W_BYTES;
         if (!idle) {
@@ -129,7 +127,8 @@ __device__ __forceinline__ void xm_body(const XmSlab &sl, const uint16_t *x, con
                         acc[cb][tb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cb], b[tb], acc[cb][tb], 0, 0, 0);
             }
         }
-        buf = buf + 1 == XM_NBUF ? 0 : buf + 1;
+        buf ^= 1;
+        __syncthreads();                                           // the buffer may be requested into again
     }
     // accumulator register r of lane (token, half) is column 8*(r/4) + 4*half + r%4 of its 32-column block
     if (!idle) {
