@@ -302,6 +302,51 @@ def other_shapes_leg(torch, pypto_amd, dev):
     return res
 
 
+def prefill_prologs_leg(torch, pypto_amd, dev):
+    """The two prologs at the reference's prefill-sized cases (MLA prolog b=1 s=512; indexer prolog b=128 s=4 and
+    b=1 s=4096): time per eager call, in the default summation mode and with the indexer's sums over the hidden
+    axis on the matrix cores."""
+    from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
+    from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
+
+    def timed(fn, n=10):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+    res = []
+    d = gen_mla_prolog_inputs(1, 512, [4096], seed=0).to(dev)
+    t, n, ql = 512, 128, 1536
+    outs = (torch.empty([t, ql], dtype=torch.int8, device=dev), torch.empty([t, 1], dtype=torch.float32, device=dev),
+            torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev), torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev),
+            d.kv_cache, d.kr_cache, d.k_scale_cache)
+    ins = list(d.input_tensors())
+    res.append({"operator": "mla_prolog_quant_p", "tokens": t, "sums": "default",
+                "us_per_call": timed(lambda: pypto_amd.mla_prolog_quant_p(*ins, *outs, 1e-5, 1e-5, "PA_BSND", None, None))})
+    del d, outs, ins
+    for b, s1, act in ((128, 4, [8192] * 128), (1, 4096, [65536])):
+        d = gen_indexer_prolog_inputs(b, s1, act, seed=0).to(dev)
+        t, n = b * s1, d.w_proj.shape[1]
+        outs = (torch.empty([t, n, 128], dtype=torch.int8, device=dev), torch.empty([t, n, 1], dtype=torch.float16, device=dev),
+                d.k_cache, d.k_cache_scale, torch.empty([t, n], dtype=torch.float16, device=dev))
+        ins = list(d.input_tensors())
+        for mode in ("default", "hidden-axis sums on the matrix cores"):
+            lip_impl.MATRIX_CORE_HIDDEN_SUMS = mode != "default"
+            try:
+                us = timed(lambda: pypto_amd.lightning_indexer_prolog_quant(*ins, *outs))
+            finally:
+                lip_impl.MATRIX_CORE_HIDDEN_SUMS = False
+            res.append({"operator": "lightning_indexer_prolog_quant", "tokens": t, "sums": mode, "us_per_call": us})
+        del d, outs, ins
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -315,6 +360,9 @@ def main():
     ap.add_argument("--other-shapes", action="store_true",
                     help="also time configs[3] (B=64, two query tokens) and configs[4] (4096-token prefill chunk) "
                          "and add them to the JSON line as 'other_shapes'")
+    ap.add_argument("--prefill-prologs", action="store_true",
+                    help="also time the MLA prolog at 512 tokens and the indexer prolog at 512 and 4096 tokens "
+                         "and add them to the JSON line as 'prefill_prologs'")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path is built and measured on ONE GPU; run with --gpus 1 "
@@ -542,6 +590,8 @@ def main():
     }
     if args.other_shapes:
         line["other_shapes"] = other_shapes_leg(torch, pypto_amd, dev)
+    if args.prefill_prologs:
+        line["prefill_prologs"] = prefill_prologs_leg(torch, pypto_amd, dev)
     print(json.dumps(line))
 
 

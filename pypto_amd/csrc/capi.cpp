@@ -331,7 +331,7 @@ extern "C" {
 
 const char *pto_last_error(void) { return g_err; }
 
-const char *pto_version(void) { return "0.4.0"; }
+const char *pto_version(void) { return "0.5.0"; }
 
 int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
 {
