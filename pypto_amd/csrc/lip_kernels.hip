@@ -154,7 +154,7 @@ __global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][r] = 0;
 
-    const QProj qp = {p.q_norm, p.w_qb, p.qpart, p.T, p.q_lora, p.n_heads};
+    const QProj qp = {p.q_norm, p.w_qb, p.qpart, p.T, p.q_lora, p.n_heads, p.q_norm_scale, p.w_qb_scale};
     if (qwave) {
         q_half_job<HS>(qp, region, job, w, acc);
         if (w == 1) q_pair_park(region, l, acc);
@@ -216,6 +216,12 @@ __global__ __launch_bounds__(64 * QFP_WAVES) void lip_finish_query_prefill_kerne
     lip_finish_query_prefill_body(p, (int)blockIdx.x, (int)gridDim.x, lds);
 }
 
+__global__ __launch_bounds__(512) void lip_qproj_prefill256_kernel(const QProj p, const int njobs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[QP2_LDS];
+    q_prefill256_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second launch: prolog_finish.h.
 __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
@@ -237,9 +243,16 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
     const int q_jobs = unsplit ? 0 : p.n_heads * LIP_KSPLIT * tblocks;
     if (unsplit) {
         if (p.q_lora % (32 * QPF_STEPS)) return hipErrorInvalidValue;
-        const QProj qp = {p.q_norm, p.w_qb, p.qpart, p.T, p.q_lora, p.n_heads};
-        const int njobs = q_prefill_jobs(qp);
-        hipLaunchKernelGGL(lip_qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+        const QProj qp = {p.q_norm, p.w_qb, p.qpart, p.T, p.q_lora, p.n_heads, p.q_norm_scale, p.w_qb_scale};
+        const int cus = cu_count();
+        if (cus <= 0) return hipErrorNoDevice;
+        const int njobs256 = q_prefill256_jobs(qp);
+        if (4 * njobs256 >= 3 * cus) {                // enough 256 x 256 tiles to fill the chip
+            hipLaunchKernelGGL(lip_qproj_prefill256_kernel, dim3((unsigned)njobs256), dim3(512), 0, stream, qp, njobs256);
+        } else {
+            const int njobs = q_prefill_jobs(qp);
+            hipLaunchKernelGGL(lip_qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+        }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -247,6 +247,12 @@ __global__ __launch_bounds__(256) void qproj_prefill_kernel(const QProj p, const
     q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
+__global__ __launch_bounds__(512) void qproj_prefill256_kernel(const QProj p, const int njobs)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[QP2_LDS];
+    q_prefill256_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Last launch: prolog_finish.h.
 __global__ __launch_bounds__(256) void mlap_finish_kernel(const MlapParams p)
@@ -308,9 +314,16 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
     hipLaunchKernelGGL(mlap_mid_kernel, dim3((unsigned)(2 * p.T)), dim3(64 * MID_WAVES), 0, stream, p, ngroups);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128};
+    const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128, p.q_norm_scale, p.w_qb_scale};
     if (qproj_splits(p.T) == 1) {
         if (p.q_lora % (32 * QPF_STEPS)) return hipErrorInvalidValue;
+        const int cus = cu_count();
+        if (cus <= 0) return hipErrorNoDevice;
+        const int njobs256 = q_prefill256_jobs(qp);
+        if (4 * njobs256 >= 3 * cus) {                 // enough 256 x 256 tiles to fill the chip
+            hipLaunchKernelGGL(qproj_prefill256_kernel, dim3((unsigned)njobs256), dim3(512), 0, stream, qp, njobs256);
+            return hipGetLastError();
+        }
         const int njobs = q_prefill_jobs(qp);
         hipLaunchKernelGGL(qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
         return hipGetLastError();

@@ -16,8 +16,12 @@ __host__ __device__ inline int qproj_splits(const int T) { return T >= QPROJ_PRE
 struct QProj {
     const int8_t *q_norm;   // [T, q_lora]
     const int8_t *w;        // [q_lora, 128 * nslabs], row-major
-    int32_t *part;          // [qproj_splits(T), T, 128 * nslabs]
+    int32_t *part;          // split form: int32 partial sums [QPROJ_KSPLIT, T, 128 * nslabs]; unsplit form: the
+                            // de-quantised results as bf16 [T, 128 * nslabs] (half the bytes on their way to the
+                            // last launch, which would de-quantise them first thing anyway)
     int T, q_lora, nslabs;
+    const float *tok_scale; // [T]              } result = bf16((float(sum) * tok_scale[t]) * col_scale[column]),
+    const float *col_scale; // [128 * nslabs]   } read by the unsplit form only
 };
 
 #define VM_WAIT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | (((n) >> 4) << 14) | 0x0F70))
@@ -107,7 +111,8 @@ __device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const i
 // read rows 0..15 of the step, lanes 32..63 rows 16..31; a row is 32 dwords, so rows of the same parity share their
 // banks: rows 16..31 sit in LDS with neighbours swapped (row 16 + r at 16 + (r ^ 1)), which puts the two half-waves
 // of a read on opposite halves of the banks.
-__device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *tok, const int s, const int l, i32x16 (&acc)[4])
+// the four weight operands of step s (32 output columns each) from the tile
+__device__ __forceinline__ void q_build_a(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
 {
     const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(tile);
     const int hi = l >> 5;
@@ -116,8 +121,6 @@ __device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *to
     uint32_t d[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + ((r & 1) ? rd_odd : rd_even) + r * 32];
-    const i32x4 b = *reinterpret_cast<const i32x4 *>(tok + 1024 * s + 16 * l);
-    i32x4 a[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
         uint32_t o0, o1, o2, o3;
@@ -127,6 +130,12 @@ __device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *to
         a[2][q] = (int)o2;
         a[3][q] = (int)o3;
     }
+}
+__device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *tok, const int s, const int l, i32x16 (&acc)[4])
+{
+    i32x4 a[4];
+    q_build_a(tile, s, l, a);
+    const i32x4 b = *reinterpret_cast<const i32x4 *>(tok + 1024 * s + 16 * l);
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
 }
@@ -197,6 +206,40 @@ __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const 
     }
 }
 
+// The unsplit forms' results leave de-quantised, as bf16, through a staging area of the wave's own in LDS
+// (Q_STAGE_BYTES; the chunk buffers are free by then), so that they reach memory as whole 256-byte rows instead of
+// 8-byte fragments of 32 different rows: accumulator register r of the four products holds columns 4m .. 4m+3 of this
+// lane's token (m as in q_pair_store_from).  tbase: first of the wave's 32 tokens; col0: first of its 128 columns.
+constexpr int Q_STAGE_PITCH = 272;                     // bytes between token rows: 16-byte aligned, 4 banks apart
+constexpr int Q_STAGE_BYTES = 32 * Q_STAGE_PITCH;
+__device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16 (&acc)[4], const int tbase, const int col0, const int l,
+                                                    uint8_t *stage)
+{
+    const int ncols = p.nslabs * 128;
+    const int t = tbase + (l & 31);
+    const float ts = p.tok_scale[t < p.T ? t : p.T - 1];
+    const float *cs = p.col_scale + col0;
+    uint8_t *mine = stage + (l & 31) * Q_STAGE_PITCH;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
+        const f32x4 c = *reinterpret_cast<const f32x4 *>(cs + 4 * m);
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __fmul_rn(__fmul_rn((float)acc[i][r], ts), c[i]);
+        const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        *reinterpret_cast<u32x2 *>(mine + 8 * m) = o;
+    }
+    // the wave reads back what it wrote itself: LDS operations of a wave stay in order
+    uint16_t *dst = reinterpret_cast<uint16_t *>(p.part) + col0 + 8 * (l & 15);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int row = 4 * k + (l >> 4);
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * Q_STAGE_PITCH + 16 * (l & 15));
+        if (tbase + row < p.T) *reinterpret_cast<u32x4 *>(dst + (size_t)(tbase + row) * ncols) = v;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // The projection at prefill sizes (T >= QPROJ_PREFILL_TOKENS): one workgroup of four waves per (slab of 128
 // columns, block of 128 tokens) walks the whole reduction axis in chunks of 128 rows, so a weight tile is read
@@ -252,16 +295,96 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
         for (int s = 0; s < QPF_STEPS; ++s) q_step_at(buf, buf + QPF_TILE + w * QPF_TOK, s, l, acc);
         __syncthreads();                               // chunk c + 2 goes where chunk c was read
     }
-    if (t < p.T) {
-        int32_t *dst = p.part + (size_t)t * ncols + slab * 128;
+    static_assert(4 * Q_STAGE_BYTES <= QPF_LDS, "the staging areas reuse the chunk buffers");
+    q_store_dequantised(p, acc, t - (l & 31), slab * 128, l, lds + w * Q_STAGE_BYTES);   // past the loop's last barrier
+}
+// The same projection for grids that fill the chip with larger tiles: a workgroup of eight waves per (256 columns,
+// 256 tokens); wave (wc, wt) holds columns 128*wc .. +127 x tokens 64*wt .. +63 (eight accumulators), so a weight
+// operand built from LDS serves two token blocks and every byte staged serves four times the products of the
+// 128 x 128 form -- these kernels are bound by the operand traffic from the L2 into LDS, not by the matrix cores.
+// Chunks of 64 rows (two steps): the tile as two halves of [64 rows][128 bytes] and the token operands of eight
+// token blocks x two steps, 32 KiB, in three buffers two chunks ahead of the products; one barrier per chunk.
+constexpr int QP2_BUF = 2 * 64 * 128 + 16 * 1024;
+constexpr int QP2_NBUF = 3;
+constexpr int QP2_LDS = QP2_NBUF * QP2_BUF;            // 96 KiB
+
+__host__ __device__ inline int q_prefill256_jobs(const QProj &p) { return ((p.nslabs + 1) / 2) * ((p.T + 255) / 256); }
+
+__device__ __forceinline__ void q_prefill256_body(const QProj &p, const int job, uint8_t *lds)
+{
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wc = w & 1, wt = w >> 1;
+    const int ncols = p.nslabs * 128;
+    const int ttiles = (p.T + 255) / 256;
+    const int ct = job / ttiles;
+    const int t0 = (job % ttiles) * 256;
+    const int nch = p.q_lora / 64;
+    const bool cols_live = 2 * ct + wc < p.nslabs;      // an odd number of slabs leaves the last tile half empty
+    const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
+    // this wave's four requests of a chunk: tile pieces 2w, 2w+1 (half = piece / 8; rows 8*(piece % 8) .. +7 of the
+    // chunk, neighbours swapped in rows 16..31 of a step) and token pieces 2w, 2w+1 (token block w, steps 0 and 1)
+    const int8_t *tsrc[2];
+    uint32_t tdst[2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
-            const i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-            *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
+    for (int j = 0; j < 2; ++j) {
+        const int q = 2 * w + j;
+        const int half = q >> 3, rb = q & 7;
+        const int slab = 2 * ct + half < p.nslabs ? 2 * ct + half : p.nslabs - 1;
+        const int row = 8 * rb + (((rb & 3) >= 2) ? ((l >> 3) ^ 1) : (l >> 3));
+        tsrc[j] = p.w + (size_t)row * ncols + slab * 128 + 16 * (l & 7);
+        tdst[j] = half * 8192 + rb * 1024;
+    }
+    int t = t0 + 32 * w + (l & 31);
+    t = t < p.T ? t : p.T - 1;
+    const int8_t *ksrc = p.q_norm + (size_t)t * p.q_lora + 16 * (l >> 5);
+    auto issue = [&](const int c, const int buf) {
+        const uint32_t b = base + buf * QP2_BUF;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) dma16(tsrc[j] + (size_t)c * 64 * ncols, b + tdst[j]);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) dma16(ksrc + c * 64 + 32 * s, b + 16384 + (2 * w + s) * 1024);
+    };
+    i32x16 acc[2][4];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[tb][i][r] = 0;
+    issue(0, 0);
+    if (nch > 1) issue(1, 1);
+    int buf = 0;
+#pragma unroll 1
+    for (int c = 0; c < nch; ++c) {
+        if (c + 1 < nch) VM_WAIT(4);
+        else VM_WAIT(0);
+        __syncthreads();                               // chunk c has landed for every wave; every wave is done with chunk c - 1
+        if (c + 2 < nch) issue(c + 2, buf == 0 ? 2 : buf - 1);
+        const uint8_t *bp = lds + buf * QP2_BUF;
+        if (cols_live) {
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                i32x4 a[4];
+                q_build_a(bp + wc * 8192, s, l, a);
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    const i32x4 b = *reinterpret_cast<const i32x4 *>(bp + 16384 + (2 * (2 * wt + tb) + s) * 1024 + 16 * l);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[tb][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[tb][i], 0, 0, 0);
+                }
+            }
         }
+        buf = buf == 2 ? 0 : buf + 1;
+    }
+    static_assert(8 * Q_STAGE_BYTES <= QP2_LDS, "the staging areas reuse the chunk buffers");
+    __syncthreads();                                   // every wave is done with the last chunk
+    if (cols_live) {
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb) q_store_dequantised(p, acc[tb], t0 + 64 * wt + 32 * tb, (2 * ct + wc) * 128, l, lds + w * Q_STAGE_BYTES);
     }
 }
+
 // workgroup number -> job, so that the workgroups of a slab (consecutive jobs) run on one XCD (workgroups go round
 // the eight XCDs) and share its L2 copy of the weight tile
 __device__ __forceinline__ int q_prefill_job_of(const int wg, const int njobs)

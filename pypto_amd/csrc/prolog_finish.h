@@ -12,23 +12,26 @@
 namespace pto {
 namespace {
 
-// the int8 projection's result for columns col, col + 1 of token t: its partial sums added
-__device__ __forceinline__ void part_sum2(const int32_t *part, const int T, const int t, const int ncols, const int col, int &s0, int &s1)
+// the de-quantised int8 projection for columns col, col + 1 of token t, as bf16-valued floats: the unsplit form left
+// them that way; the split form's partial sums are added and de-quantised here
+__device__ __forceinline__ void q_value2(const int32_t *part, const int T, const int t, const int ncols, const int col, const float ts,
+                                         const float cs0, const float cs1, float &v0, float &v1)
 {
     if (qproj_splits(T) == 1) {
-        const int2 v = *reinterpret_cast<const int2 *>(part + (size_t)t * ncols + col);
-        s0 = v.x;
-        s1 = v.y;
+        const uint32_t v = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(part) + (size_t)t * ncols + col);
+        v0 = __uint_as_float(v << 16);
+        v1 = __uint_as_float(v & 0xffff0000u);
         return;
     }
-    s0 = 0;
-    s1 = 0;
+    int s0 = 0, s1 = 0;
 #pragma unroll
     for (int kq = 0; kq < QPROJ_KSPLIT; ++kq) {
         const int2 v = *reinterpret_cast<const int2 *>(part + ((size_t)kq * T + t) * ncols + col);
         s0 += v.x;
         s1 += v.y;
     }
+    v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs0));
+    v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs1));
 }
 
 // ------------------------------------------------------------------------------ indexer prolog
@@ -141,13 +144,11 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
         const int t = live ? row / p.n_heads : 0;
         const int head = live ? row % p.n_heads : 0;
         const int col = head * LIP_DIM + 2 * l;
-        int s0, s1;
-        part_sum2(p.qpart, p.T, t, ncols, col, s0, s1);
         const float ts = p.q_norm_scale[t];
         const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
         const uint32_t rc = rope_coef(p.cos, t, l), rs = rope_coef(p.sin, t, l);
-        float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
-        float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
+        float v0, v1;
+        q_value2(p.qpart, p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
         rope_pair(v0, v1, rc, rs, l);
         f32x2 av = {v0, v1};
         *reinterpret_cast<f32x2 *>(&arow[w][2 * l]) = av;
@@ -288,9 +289,7 @@ __device__ __forceinline__ void lip_finish_query_prefill_body(const LipParams &p
     for (int pass = wg * QFP_WAVES + w; pass < npass; pass += nwg * QFP_WAVES) {
 #pragma unroll 1
         for (int b8 = 0; b8 < 4; ++b8) {
-            int2 raw[8];
-            float ts[8];
-            f32x2 cs[8];
+            uint32_t raw[8];
             uint32_t rc[8], rs[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
@@ -298,16 +297,14 @@ __device__ __forceinline__ void lip_finish_query_prefill_body(const LipParams &p
                 const int rr = row < nrows ? row : nrows - 1;
                 const int t = rr / p.n_heads;
                 const int col = (rr - t * p.n_heads) * LIP_DIM + 2 * l;
-                raw[u] = *reinterpret_cast<const int2 *>(p.qpart + (size_t)t * ncols + col);
-                ts[u] = p.q_norm_scale[t];
-                cs[u] = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
+                raw[u] = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(p.qpart) + (size_t)t * ncols + col);
                 rc[u] = rope_coef(p.cos, t, l);
                 rs[u] = rope_coef(p.sin, t, l);
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
-                float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw[u].x, ts[u]), cs[u][0]));
-                float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw[u].y, ts[u]), cs[u][1]));
+                float v0 = __uint_as_float(raw[u] << 16);      // the unsplit projection leaves its results de-quantised
+                float v1 = __uint_as_float(raw[u] & 0xffff0000u);
                 rope_pair(v0, v1, rc[u], rs[u], l);
                 *reinterpret_cast<uint32_t *>(abf + (b8 * 8 + u) * QFP_APITCH + 2 * l) = pack_bf16x2(v0, v1);
             }
@@ -407,22 +404,19 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
         // nope part: lane l -> channels 2l, 2l+1
         {
             const int col = head * MLAP_QHEAD + 2 * l;
-            int s0, s1;
-            part_sum2(p.qpart, p.T, tt, ncols, col, s0, s1);
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
-            f32x2 av = {bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0])),
-                        bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]))};
+            float av0, av1;
+            q_value2(p.qpart, p.T, tt, ncols, col, ts, cs[0], cs[1], av0, av1);
+            const f32x2 av = {av0, av1};
             *reinterpret_cast<f32x2 *>(&arow[tl][2 * l]) = av;
             *reinterpret_cast<uint32_t *>(&abf[tl][2 * l]) = pack_bf16x2(av[0], av[1]);
         }
         // rope part (first half-workgroup only): lane l < 32 -> channels 2l, 2l+1 = rotation partners l, 32+l
         if (half == 0 && l < 32 && t < p.T) {
             const int col = head * MLAP_QHEAD + MLAP_NOPE + 2 * l;
-            int s0, s1;
-            part_sum2(p.qpart, p.T, t, ncols, col, s0, s1);
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
-            const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s0, ts), cs[0]));
-            const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)s1, ts), cs[1]));
+            float v0, v1;
+            q_value2(p.qpart, p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
             const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
             const float sn0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), sn1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
             const float r0 = __builtin_fmaf(v0, c0, (-v1) * sn0);
@@ -519,8 +513,8 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
 // The same last stage for 64 tokens and more with the absorb product on the matrix cores: one workgroup of eight
 // waves per (head, run of `per` blocks of 32 tokens).  The head's whole w_uk (128 x 512 bf16, 128 KiB) is staged
 // once, wave w keeping the slice of output columns 64w..64w+63 in the layout of the decode form; then per block:
-// wave w de-quantises the query channels of tokens 4w..4w+3 (the projection is unsplit at these sizes) into one of two
-// bf16 operand buffers and rotates and stores their rope part, the loads of the next block go out, one barrier, and
+// wave w moves the query channels of tokens 4w..4w+3 (de-quantised bf16 already: the projection is unsplit at these
+// sizes) into one of two bf16 operand buffers and rotates and stores their rope part, the loads of the next block go out, one barrier, and
 // 16 products per wave give 32 tokens x 64 columns.  A weight slice is read once per `per` blocks instead of once
 // per 8 tokens; each output has the bits of the decode form (same products, same order).
 constexpr int FINP_TOK = 32;
@@ -530,8 +524,7 @@ constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_API
 static_assert(MLAP_MFMA_MIN_TOKENS >= QPROJ_PREFILL_TOKENS, "the prefill form reads one partial sum per output");
 
 struct FinRaw {
-    int2 nope[4], rope[4];
-    float ts[4];
+    uint32_t nope[4], rope[4];     // two bf16 values each: the unsplit projection leaves its results de-quantised
     uint16_t c0[4], c1[4], s0[4], s1[4];
 };
 
@@ -561,11 +554,10 @@ __device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, co
         for (int u = 0; u < 4; ++u) {
             const int t = blk * FINP_TOK + 4 * w + u;
             const int tt = t < p.T ? t : p.T - 1;
-            const int32_t *row = p.qpart + (size_t)tt * ncols + head * MLAP_QHEAD;
-            r.ts[u] = p.q_norm_scale[tt];
-            r.nope[u] = *reinterpret_cast<const int2 *>(row + 2 * l);
+            const uint16_t *row = reinterpret_cast<const uint16_t *>(p.qpart) + (size_t)tt * ncols + head * MLAP_QHEAD;
+            r.nope[u] = *reinterpret_cast<const uint32_t *>(row + 2 * l);
             if (l < 32) {
-                r.rope[u] = *reinterpret_cast<const int2 *>(row + MLAP_NOPE + 2 * l);
+                r.rope[u] = *reinterpret_cast<const uint32_t *>(row + MLAP_NOPE + 2 * l);
                 r.c0[u] = p.cos[(size_t)tt * MLAP_ROPE + l];
                 r.c1[u] = p.cos[(size_t)tt * MLAP_ROPE + 32 + l];
                 r.s0[u] = p.sin[(size_t)tt * MLAP_ROPE + l];
@@ -573,8 +565,6 @@ __device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, co
             }
         }
     };
-    const f32x2 cs_nope = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + head * MLAP_QHEAD + 2 * l);
-    const f32x2 cs_rope = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + head * MLAP_QHEAD + MLAP_NOPE + 2 * (l & 31));
     FinRaw raw;
     if (b0 < b1) load(raw, b0);
     VM_WAIT(0);
@@ -588,13 +578,10 @@ __device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, co
         for (int u = 0; u < 4; ++u) {
             const int tl = 4 * w + u;
             const int t = blk * FINP_TOK + tl;
-            const float ts = raw.ts[u];
-            const float a0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.nope[u].x, ts), cs_nope[0]));
-            const float a1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.nope[u].y, ts), cs_nope[1]));
-            *reinterpret_cast<uint32_t *>(&abf[buf][tl][2 * l]) = pack_bf16x2(a0, a1);
+            *reinterpret_cast<uint32_t *>(&abf[buf][tl][2 * l]) = raw.nope[u];
             if (l < 32 && t < p.T) {
-                const float v0 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.rope[u].x, ts), cs_rope[0]));
-                const float v1 = bf16_round_f32(__fmul_rn(__fmul_rn((float)raw.rope[u].y, ts), cs_rope[1]));
+                const float v0 = __uint_as_float(raw.rope[u] << 16);
+                const float v1 = __uint_as_float(raw.rope[u] & 0xffff0000u);
                 const float r0 = __builtin_fmaf(v0, bf16_bits_to_f32(raw.c0[u]), (-v1) * bf16_bits_to_f32(raw.s0[u]));
                 const float r1 = __builtin_fmaf(v1, bf16_bits_to_f32(raw.c1[u]), v0 * bf16_bits_to_f32(raw.s1[u]));
                 uint16_t *out = p.q_rope + ((size_t)t * p.n_heads + head) * MLAP_ROPE;

@@ -124,6 +124,14 @@ def test_prolog_reference_large_cases(b, s1, act, what):
     assert_exact(run_op(inp), ref, what)
 
 
+def test_prolog_large_tile_projection_ragged_tokens_odd_slab_count():
+    """1500 tokens x 63 heads: enough 256 x 256 tiles of the int8 projection to fill the chip, so that form runs, with
+    a ragged last token tile (1500 = 5 x 256 + 220) and a last column tile of which only one half exists."""
+    inp = gen_indexer_prolog_inputs(1, 1500, [3000], seed=9, h=128, q_lora_rank=512, n_heads=63)
+    ref = lo.indexer_prolog_ref(*inp.input_tensors())
+    assert_exact(run_op(inp), ref, "t1500_n63")
+
+
 PREFILL_CASES = [
     (3, 50, [700, 650, 600], dict(h=256, q_lora_rank=512, n_heads=8)),     # 150 tokens: ragged token tiles, one piece of w_proj per row
     (1, 77, [300], dict(h=192, q_lora_rank=1024, n_heads=24)),             # three chunks of the hidden axis, ragged row passes
