@@ -520,7 +520,9 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
 constexpr int FINP_TOK = 32;
 constexpr int FINP_WAVES = 8;
 constexpr int FINP_APITCH = MLAP_NOPE + 8;   // elements between operand rows: 272 bytes, so that the 32 rows of an operand read spread over the banks
-constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_APITCH * 2;   // 148 480 bytes
+constexpr int FINP_SPITCH = 144;             // bytes between the rows of a wave's output staging area (8 tokens x 64 columns)
+constexpr int FINP_STAGE = 8 * FINP_SPITCH;
+constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_APITCH * 2 + FINP_WAVES * FINP_STAGE;   // 157 696 bytes
 static_assert(MLAP_MFMA_MIN_TOKENS >= QPROJ_PREFILL_TOKENS, "the prefill form reads one partial sum per output");
 
 struct FinRaw {
@@ -611,16 +613,25 @@ __device__ __forceinline__ void mlap_finish_prefill_body(const MlapParams &p, co
                 c[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, bq), c[cb], 0, 0, 0);
             }
         }
-        const int t = blk * FINP_TOK + (l & 31);
-        if (t < p.T) {
-            uint16_t *dst = p.q_nope + ((size_t)t * p.n_heads + head) * MLAP_KV + colbase + 4 * (l >> 5);
+        // Lane (token, half) holds 8-byte fragments of its token's row; they leave through the wave's staging area,
+        // eight tokens at a time, as whole 128-byte rows (16 bytes per lane) -- scattered fragments cost the memory
+        // side several times their bytes.
+        uint8_t *stg = lds + FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_APITCH * 2 + w * FINP_STAGE;
 #pragma unroll
-            for (int cb = 0; cb < 2; ++cb)
+        for (int qt = 0; qt < 4; ++qt) {
+            if (((l & 31) >> 3) == qt) {
+                uint8_t *row = stg + (l & 7) * FINP_SPITCH + 8 * (l >> 5);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const u32x2 v = {pack_bf16x2(c[cb][4 * q], c[cb][4 * q + 1]), pack_bf16x2(c[cb][4 * q + 2], c[cb][4 * q + 3])};
-                    *reinterpret_cast<u32x2 *>(dst + 32 * cb + 8 * q) = v;
-                }
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const u32x2 v = {pack_bf16x2(c[cb][4 * q], c[cb][4 * q + 1]), pack_bf16x2(c[cb][4 * q + 2], c[cb][4 * q + 3])};
+                        *reinterpret_cast<u32x2 *>(row + 64 * cb + 16 * q) = v;
+                    }
+            }
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(stg + (l >> 3) * FINP_SPITCH + 16 * (l & 7));
+            const int t = blk * FINP_TOK + 8 * qt + (l >> 3);
+            if (t < p.T) *reinterpret_cast<u32x4 *>(p.q_nope + ((size_t)t * p.n_heads + head) * MLAP_KV + colbase + 8 * (l & 7)) = v;
         }
     }
 }

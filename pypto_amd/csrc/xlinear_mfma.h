@@ -26,6 +26,7 @@ constexpr int XM_W_BYTES = XM_KC * 256;          // slab rows are staged 256 byt
 constexpr int XM_X_BYTES = XM_TOK * XM_KC * 2;
 constexpr int XM_BUF = XM_W_BYTES + XM_X_BYTES;
 constexpr int XM_LDS = 2 * XM_BUF;
+constexpr int XM_SPITCH = 272;                   // bytes between the rows of a wave's output staging area (32 tokens x 64 columns fp32)
 
 struct XmSlab {
     const uint8_t *w;     // column 0 of the slab in row 0 of the weight matrix
@@ -130,23 +131,30 @@ __device__ __forceinline__ void xm_body(const XmSlab &sl, const uint16_t *x, con
         buf ^= 1;
         __syncthreads();                                           // the buffer may be requested into again
     }
-    // accumulator register r of lane (token, half) is column 8*(r/4) + 4*half + r%4 of its 32-column block
+    // accumulator register r of lane (token, half) is column 8*(r/4) + 4*half + r%4 of its 32-column block: 16-byte
+    // fragments of 32 different rows per store; they leave through a staging area of the wave's own (the chunk
+    // buffers are free past the loop's last barrier) as whole 256-byte row segments instead
+    static_assert(4 * 32 * XM_SPITCH <= XM_LDS, "the staging areas reuse the chunk buffers");
     if (!idle) {
+        uint8_t *stg = smem + w * (32 * XM_SPITCH);
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb) {
-            const int t = t0 + 64 * wt + 32 * tb + (l & 31);
-            if (t < T) {
-                const int col0 = 64 * wc + 4 * (l >> 5);
-                float *dst = sl.out + (size_t)t * sl.out_pitch + col0;
+            uint8_t *row = stg + (l & 31) * XM_SPITCH + 16 * (l >> 5);
 #pragma unroll
-                for (int cb = 0; cb < 2; ++cb)
+            for (int cb = 0; cb < 2; ++cb)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if (col0 + 32 * cb + 8 * q < 8 * sl.pieces) {
-                            const f32x4 v = {acc[cb][tb][4 * q], acc[cb][tb][4 * q + 1], acc[cb][tb][4 * q + 2], acc[cb][tb][4 * q + 3]};
-                            *reinterpret_cast<f32x4 *>(dst + 32 * cb + 8 * q) = v;
-                        }
-                    }
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v = {acc[cb][tb][4 * q], acc[cb][tb][4 * q + 1], acc[cb][tb][4 * q + 2], acc[cb][tb][4 * q + 3]};
+                    *reinterpret_cast<f32x4 *>(row + 128 * cb + 32 * q) = v;
+                }
+            // the wave reads back what it wrote itself: LDS operations of a wave stay in order
+            const int col = 64 * wc + 4 * (l & 15);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int r = 4 * k + (l >> 4);
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(stg + r * XM_SPITCH + 16 * (l & 15));
+                const int t = t0 + 64 * wt + 32 * tb + r;
+                if (t < T && col < 8 * sl.pieces) *reinterpret_cast<f32x4 *>(sl.out + (size_t)t * sl.out_pitch + col) = v;
             }
         }
     }
