@@ -222,6 +222,12 @@ __global__ __launch_bounds__(512) void lip_qproj_prefill256_kernel(const QProj p
     q_prefill256_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
+__global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_tokens_prefill_kernel(const LipParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LIP_FINT_LDS];
+    lip_finish_tokens_prefill_body(p, (int)blockIdx.x, lds);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second launch: prolog_finish.h.
 __global__ __launch_bounds__(64 * FIN_WAVES) void lip_finish_kernel(const LipParams p, const int q_wgs)
@@ -303,6 +309,9 @@ hipError_t lip_launch_finish(const LipParams &p, hipStream_t stream)
         hipLaunchKernelGGL(lip_finish_query_prefill_kernel, dim3((unsigned)wgs), dim3(64 * QFP_WAVES), 0, stream, p);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+        // key rows and weights: eight tokens per workgroup
+        hipLaunchKernelGGL(lip_finish_tokens_prefill_kernel, dim3((unsigned)((p.T + FIN_WAVES - 1) / FIN_WAVES)), dim3(64 * FIN_WAVES), 0, stream, p);
+        return hipGetLastError();
     }
     hipLaunchKernelGGL(lip_finish_kernel, dim3((unsigned)(q_wgs + p.T)), dim3(64 * FIN_WAVES), 0, stream, p, q_wgs);
     return hipGetLastError();

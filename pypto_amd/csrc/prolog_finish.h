@@ -121,6 +121,36 @@ __device__ __forceinline__ void stage_matrix(uint16_t *dst, const uint16_t *src)
     for (int i = 0; i < 2048 / NT; ++i) d[i * NT + threadIdx.x] = s[i * NT + threadIdx.x];
 }
 
+// a key row from its sums over the hidden axis (lane l: channels 2l, 2l+1): layer norm, rope, Hadamard product with the
+// matrix in LDS (a: this wave's 128 floats of LDS), quantisation, scatter to cache row dst (skipped if out of range)
+__device__ __forceinline__ void lip_key_row(const LipParams &p, const uint16_t *hmat, float *a, float v0, float v1, const uint32_t rc,
+                                            const uint32_t rs, const uint32_t gm, const uint32_t bt, const long long dst, const int l)
+{
+    const float mean = __fmul_rn(pair_tree_sum(v0, v1), 1.0f / LIP_DIM);
+    const float d0 = __fsub_rn(v0, mean), d1 = __fsub_rn(v1, mean);
+    const float var = __fmul_rn(pair_tree_sum(__fmul_rn(d0, d0), __fmul_rn(d1, d1)), 1.0f / LIP_DIM);
+    const float sd = __builtin_sqrtf(__fadd_rn(var, p.eps));   // correctly rounded (__fsqrt_rn is the 1-ulp hardware root here)
+    v0 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d0, sd), __uint_as_float(gm << 16)), __uint_as_float(bt << 16)));
+    v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(gm & 0xffff0000u)), __uint_as_float(bt & 0xffff0000u)));
+    rope_pair(v0, v1, rc, rs, l);
+    f32x2 av = {v0, v1};
+    *reinterpret_cast<f32x2 *>(&a[2 * l]) = av;
+    float y0, y1;
+    hadamard_pair(a, hmat, l, y0, y1);                 // the same wave wrote a: LDS operations of a wave stay in order
+    uint16_t sc;
+    const uint16_t q = quant_pair(y0, y1, sc);
+    if (dst >= 0 && dst < p.cache_rows) {
+        reinterpret_cast<uint16_t *>(p.k_cache + (size_t)dst * LIP_DIM)[l] = q;
+        if (l == 0) p.k_cache_scale[dst] = sc;
+    }
+}
+// head weight l of token t from its sum over the hidden axis
+__device__ __forceinline__ void lip_weight(const LipParams &p, const int t, const int l, float v)
+{
+    v = __fmul_rn(__fmul_rn(bf16_round_f32(v), p.w_mul0), p.w_mul1);
+    p.weights[(size_t)t * p.n_heads + l] = (uint16_t)(pack_f16x2(v, 0.f) & 0xffffu);
+}
+
 // Workgroups [0, q_wgs): FIN_WAVES query rows (token, head) each, one per wave.
 // Workgroups [q_wgs, q_wgs + T): one token each -- waves add the groups of block sums over the hidden
 // axis (two groups of eight blocks per wave and round), then wave 0 finishes the key row and wave 1 the
@@ -225,30 +255,77 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
             v0 = __fadd_rn(v0, v[0]);
             v1 = __fadd_rn(v1, v[1]);
         }
-        // layer norm over the 128 channels
-        const float mean = __fmul_rn(pair_tree_sum(v0, v1), 1.0f / LIP_DIM);
-        const float d0 = __fsub_rn(v0, mean), d1 = __fsub_rn(v1, mean);
-        const float var = __fmul_rn(pair_tree_sum(__fmul_rn(d0, d0), __fmul_rn(d1, d1)), 1.0f / LIP_DIM);
-        const float sd = __builtin_sqrtf(__fadd_rn(var, p.eps));   // correctly rounded (__fsqrt_rn is the 1-ulp hardware root here)
-        v0 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d0, sd), __uint_as_float(gm << 16)), __uint_as_float(bt << 16)));
-        v1 = bf16_round_f32(__fadd_rn(__fmul_rn(__fdiv_rn(d1, sd), __uint_as_float(gm & 0xffff0000u)), __uint_as_float(bt & 0xffff0000u)));
-        rope_pair(v0, v1, rc, rs, l);
-        f32x2 av = {v0, v1};
-        *reinterpret_cast<f32x2 *>(&arow[0][2 * l]) = av;
-        float y0, y1;
-        hadamard_pair(arow[0], hmat, l, y0, y1);       // same wave wrote arow[0]: LDS operations of a wave stay in order
-        uint16_t sc;
-        const uint16_t q = quant_pair(y0, y1, sc);
-        if (dst >= 0 && dst < p.cache_rows) {
-            reinterpret_cast<uint16_t *>(p.k_cache + (size_t)dst * LIP_DIM)[l] = q;
-            if (l == 0) p.k_cache_scale[dst] = sc;
-        }
+        lip_key_row(p, hmat, arow[0], v0, v1, rc, rs, gm, bt, dst, l);
     } else if (w == 1 && pl) {
         float v = 0.f;
         for (int g = 0; g < ngroups; ++g) v = __fadd_rn(v, gsum[g][LIP_DIM + l]);
-        v = __fmul_rn(__fmul_rn(bf16_round_f32(v), p.w_mul0), p.w_mul1);
-        p.weights[(size_t)t * p.n_heads + l] = (uint16_t)(pack_f16x2(v, 0.f) & 0xffffu);
+        lip_weight(p, t, l, v);
     }
+}
+
+// The key rows and weights at prefill sizes: a workgroup of FIN_WAVES waves takes FIN_WAVES tokens, one per wave (the
+// matrix is staged once for all of them instead of once per token, and the rows are finished side by side instead of
+// by one wave per workgroup).  A wave adds its token's partial rows in registers, in the order of the form they come
+// in: group sums ascending, or blocks / ranges ascending into groups of eight and the groups ascending.
+constexpr int LIP_FINT_LDS = LIP_DIM * LIP_DIM * 2 + FIN_WAVES * LIP_DIM * 4;
+
+__device__ __forceinline__ void lip_finish_tokens_prefill_body(const LipParams &p, const int wg, uint8_t *lds)
+{
+    uint16_t *hmat = reinterpret_cast<uint16_t *>(lds);
+    float(*arow)[LIP_DIM] = reinterpret_cast<float(*)[LIP_DIM]>(lds + LIP_DIM * LIP_DIM * 2);
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t = wg * FIN_WAVES + w;
+    const bool live = t < p.T;
+    const int tt = live ? t : p.T - 1;
+    stage_matrix(hmat, p.hk);
+    const bool pl = l < p.n_heads;
+    const uint32_t rc = rope_coef(p.cos, tt, l), rs = rope_coef(p.sin, tt, l);
+    const uint32_t gm = reinterpret_cast<const uint32_t *>(p.gamma)[l];
+    const uint32_t bt = reinterpret_cast<const uint32_t *>(p.beta)[l];
+    const long long dst = live ? p.k_cache_index[tt] : -1;
+    const bool group_rows = lip_x_group_rows(p);
+    const int nrows = lip_xrows(p);
+    const float *src = p.xpart + (size_t)tt * LIP_XCOLS;
+    const size_t rstride = (size_t)p.T * LIP_XCOLS;
+    float v0 = 0.f, v1 = 0.f, v2 = 0.f;
+    for (int g0 = 0; g0 < nrows; g0 += LIP_XGROUP) {
+        f32x2 kv[LIP_XGROUP];
+        float wv[LIP_XGROUP];
+        const int nb = nrows - g0 < LIP_XGROUP ? nrows - g0 : LIP_XGROUP;
+#pragma unroll
+        for (int i = 0; i < LIP_XGROUP; ++i) {
+            const float *r = src + (size_t)(g0 + (i < nb ? i : 0)) * rstride;
+            kv[i] = *reinterpret_cast<const f32x2 *>(r + 2 * l);
+            wv[i] = r[LIP_DIM + (pl ? l : 0)];
+        }
+        if (group_rows) {
+#pragma unroll
+            for (int i = 0; i < LIP_XGROUP; ++i) {
+                if (i < nb) {
+                    v0 = __fadd_rn(v0, kv[i][0]);
+                    v1 = __fadd_rn(v1, kv[i][1]);
+                    v2 = __fadd_rn(v2, wv[i]);
+                }
+            }
+        } else {
+            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int i = 0; i < LIP_XGROUP; ++i) {
+                if (i < nb) {
+                    s0 = __fadd_rn(s0, kv[i][0]);
+                    s1 = __fadd_rn(s1, kv[i][1]);
+                    s2 = __fadd_rn(s2, wv[i]);
+                }
+            }
+            v0 = __fadd_rn(v0, s0);
+            v1 = __fadd_rn(v1, s1);
+            v2 = __fadd_rn(v2, s2);
+        }
+    }
+    __syncthreads();                                   // the matrix is staged
+    lip_key_row(p, hmat, arow[w], v0, v1, rc, rs, gm, bt, dst, l);
+    if (pl && live) lip_weight(p, t, l, v2);
 }
 
 
