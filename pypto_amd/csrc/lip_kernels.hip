@@ -172,23 +172,24 @@ __global__ __launch_bounds__(256) void lip_qproj_prefill_kernel(const QProj p, c
     q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
-// The fixed-order sums over the hidden axis at prefill sizes (xlinear_fixed.h): workgroup = (wk or w_proj, group of
-// eight blocks, 8 tokens); only the group sums reach memory, an eighth of the rows the decode form leaves, and a
-// block of weights serves eight tokens instead of two.
+// The fixed-order sums over the hidden axis at prefill sizes (xlinear_fixed.h, the form that broadcasts the hidden
+// states through DPP): workgroup = (wk or w_proj, group of eight blocks, 16 tokens); only the group sums reach memory,
+// an eighth of the rows the decode form leaves, and a block of weights serves sixteen tokens instead of two.
 static_assert(XL_BLOCK == LIP_XBLOCK && XL_GROUP == LIP_XGROUP, "the second launch adds groups of eight blocks of 64");
 __global__ __launch_bounds__(64 * XL_WAVES) void lip_xlinear_group_kernel(const LipParams p, const int ngroups)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[XL_LDS];
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XD_LDS];
     const int slab = blockIdx.x & 1;
     const int g = (blockIdx.x >> 1) % ngroups;
-    const int t0 = ((blockIdx.x >> 1) / ngroups) * XL_TOK;
+    const int t0 = ((blockIdx.x >> 1) / ngroups) * XD_TOK;
     XlSlab sl;
     sl.w = reinterpret_cast<const uint8_t *>(slab ? p.w_proj : p.wk);
     sl.pitch = (slab ? p.n_heads : LIP_DIM) * 2;
     sl.wbytes = sl.pitch;
     sl.out = p.xpart + (size_t)g * p.T * LIP_XCOLS + slab * LIP_DIM;
     sl.out_pitch = LIP_XCOLS;
-    xl_body(sl, p.x, p.T, p.h, g, t0, smem);
+    if (slab) xd_body<false>(sl, p.x, p.T, p.h, g, t0, smem);      // w_proj: one column per lane
+    else xd_body<true>(sl, p.x, p.T, p.h, g, t0, smem);
 }
 
 // The sums over the hidden axis on the matrix cores (xlinear_mfma.h): workgroup = (wk or w_proj, one of nsplit
@@ -270,7 +271,7 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
     }
     if (lip_x_group_rows(p)) {
         const int ngroups = lip_xrows(p);
-        const int tgroups = (p.T + XL_TOK - 1) / XL_TOK;
+        const int tgroups = (p.T + XD_TOK - 1) / XD_TOK;
         hipLaunchKernelGGL(lip_xlinear_group_kernel, dim3((unsigned)(2 * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, ngroups);
         return hipGetLastError();
     }

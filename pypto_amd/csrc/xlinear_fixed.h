@@ -114,5 +114,170 @@ __device__ __forceinline__ void xl_body(const XlSlab &sl, const uint16_t *x, con
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same sums for prefill-sized token counts with the hidden states broadcast by the multiply-add itself: a lane
+// keeps x[t][k0 + 2*(l % 16)] and x[t][k0 + 2*(l % 16) + 1] of a 32-row half block in two registers per token (every
+// row of 16 lanes holds the same 32 values), and v_fmac_f32 with the DPP control row_newbcast:n reads lane n of the
+// row, i.e. hidden row k0 + 2n (or + 1), in all lanes -- no LDS read and no extra instruction per hidden state, where
+// the form above spends an LDS broadcast of 16 bytes per four multiply-adds.  Same products, same order (a block
+// ascending from 0.0, the eight block sums ascending), so the same bits.
+//   workgroup = (slab, group of 512 hidden rows, XD_TOK tokens), eight waves, wave w takes block 8*group + w.
+//   PAIR: lane l holds columns 2l, 2l+1 (a slab of 128 columns); otherwise column l (a slab of up to 64).
+constexpr int XD_TOK = 16;
+constexpr int XD_LDS = XL_WAVES * XL_W_BYTES;
+
+// acc[t] += bcast_N(x[t]) * w for eight tokens (and a second column with w1), as one statement: nothing the compiler
+// emits can sit between the multiply-adds, and the statement opens with the two wait states a DPP read wants after a
+// write of its operand, whatever the compiler did to these registers just before.
+#define XD_F "v_fmac_f32_dpp %"
+#define XD_B " row_newbcast:%[n] row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+template <int N>
+__device__ __forceinline__ void fmac8_pair(float *a0, float *a1, const float *x, const float w0, const float w1)
+{
+    asm("s_nop 1\n\t"
+        XD_F "0, %16, %[w0]" XD_B XD_F "8, %16, %[w1]" XD_B XD_F "1, %17, %[w0]" XD_B XD_F "9, %17, %[w1]" XD_B
+        XD_F "2, %18, %[w0]" XD_B XD_F "10, %18, %[w1]" XD_B XD_F "3, %19, %[w0]" XD_B XD_F "11, %19, %[w1]" XD_B
+        XD_F "4, %20, %[w0]" XD_B XD_F "12, %20, %[w1]" XD_B XD_F "5, %21, %[w0]" XD_B XD_F "13, %21, %[w1]" XD_B
+        XD_F "6, %22, %[w0]" XD_B XD_F "14, %22, %[w1]" XD_B XD_F "7, %23, %[w0]" XD_B XD_F "15, %23, %[w1]" XD_B
+        : "+v"(a0[0]), "+v"(a0[1]), "+v"(a0[2]), "+v"(a0[3]), "+v"(a0[4]), "+v"(a0[5]), "+v"(a0[6]), "+v"(a0[7]),
+          "+v"(a1[0]), "+v"(a1[1]), "+v"(a1[2]), "+v"(a1[3]), "+v"(a1[4]), "+v"(a1[5]), "+v"(a1[6]), "+v"(a1[7])
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]), [w0] "v"(w0), [w1] "v"(w1), [n] "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void fmac8_single(float *a0, const float *x, const float w0)
+{
+    asm("s_nop 1\n\t"
+        XD_F "0, %8, %[w0]" XD_B XD_F "1, %9, %[w0]" XD_B XD_F "2, %10, %[w0]" XD_B XD_F "3, %11, %[w0]" XD_B
+        XD_F "4, %12, %[w0]" XD_B XD_F "5, %13, %[w0]" XD_B XD_F "6, %14, %[w0]" XD_B XD_F "7, %15, %[w0]" XD_B
+        : "+v"(a0[0]), "+v"(a0[1]), "+v"(a0[2]), "+v"(a0[3]), "+v"(a0[4]), "+v"(a0[5]), "+v"(a0[6]), "+v"(a0[7])
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(x[4]), "v"(x[5]), "v"(x[6]), "v"(x[7]), [w0] "v"(w0), [n] "n"(N));
+}
+#undef XD_F
+#undef XD_B
+
+template <bool PAIR, int N>
+__device__ __forceinline__ void xd_pair_of_rows(const uint8_t *wrow, const int rowbytes, const int lane_off, float (&xe)[XD_TOK],
+                                                float (&xo)[XD_TOK], float (&a0)[XD_TOK], float (&a1)[XD_TOK])
+{
+#pragma unroll
+    for (int odd = 0; odd < 2; ++odd) {
+        float *xs = odd ? xo : xe;
+        if (PAIR) {
+            const uint32_t wv = *reinterpret_cast<const uint32_t *>(wrow + (2 * N + odd) * rowbytes + lane_off);
+            const float w0 = __uint_as_float(wv << 16), w1 = __uint_as_float(wv & 0xffff0000u);
+#pragma unroll
+            for (int t = 0; t < XD_TOK; t += 8) fmac8_pair<N>(a0 + t, a1 + t, xs + t, w0, w1);
+        } else {
+            const float w0 = __uint_as_float((uint32_t) * reinterpret_cast<const uint16_t *>(wrow + (2 * N + odd) * rowbytes + lane_off) << 16);
+#pragma unroll
+            for (int t = 0; t < XD_TOK; t += 8) fmac8_single<N>(a0 + t, xs + t, w0);
+        }
+    }
+}
+
+template <bool PAIR>
+__device__ __forceinline__ void xd_body(const XlSlab &sl, const uint16_t *x, const int T, const int h, const int g, const int t0, uint8_t *smem)
+{
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nblk = h / XL_BLOCK;
+    const int wbytes = sl.wbytes;
+    const int ncols = wbytes >> 1;
+    uint8_t *region = smem + w * XL_W_BYTES;
+    const int c = g * XL_GROUP + w;                                       // this wave's block
+    const int nb = nblk - g * XL_GROUP < XL_GROUP ? nblk - g * XL_GROUP : XL_GROUP;
+    float a0[XD_TOK], a1[XD_TOK];
+#pragma unroll
+    for (int t = 0; t < XD_TOK; ++t) a0[t] = a1[t] = 0.f;
+
+    if (w < nb) {
+        const int k0 = c * XL_BLOCK;
+        const uint32_t wdst = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+        {   // rows of wbytes bytes: wbytes/16 lanes per row
+            const int lpr = wbytes >> 4;
+            const int rpi = 64 / lpr;                                     // rows per request
+            const uint8_t *src = sl.w + (size_t)(k0 + l / lpr) * sl.pitch + 16 * (l % lpr);
+#pragma unroll 1
+            for (int i = 0; i < XL_BLOCK / rpi; ++i) dma16(src + (size_t)i * rpi * sl.pitch, wdst + 1024 * i);
+        }
+        // hidden states of both half blocks: lane l holds rows k0 + 32*hb + 2*(l%16), +1 of every token
+        uint32_t xr[2][XD_TOK];
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+            for (int t = 0; t < XD_TOK; ++t) {
+                const int tt = t0 + t < T ? t0 + t : T - 1;
+                xr[hb][t] = reinterpret_cast<const uint32_t *>(x + (size_t)tt * h + k0 + 32 * hb)[l & 15];
+            }
+        VM_WAIT(0);
+        const int lane_off = PAIR ? 4 * (2 * l < ncols ? l : 0) : 2 * (l < ncols ? l : 0);
+#pragma unroll
+        for (int hb = 0; hb < 2; ++hb) {
+            float xe[XD_TOK], xo[XD_TOK];
+#pragma unroll
+            for (int t = 0; t < XD_TOK; ++t) {
+                xe[t] = __uint_as_float(xr[hb][t] << 16);
+                xo[t] = __uint_as_float(xr[hb][t] & 0xffff0000u);
+            }
+            const uint8_t *wrow = region + 32 * hb * wbytes;
+            xd_pair_of_rows<PAIR, 0>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 1>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 2>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 3>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 4>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 5>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 6>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 7>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 8>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 9>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 10>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 11>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 12>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 13>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 14>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            xd_pair_of_rows<PAIR, 15>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+        }
+    }
+    __syncthreads();                                   // every wave is done with its block of weights
+    // block sums into this wave's own (consumed) region: [XD_TOK tokens][128 columns]
+    if (w < nb) {
+        float *bs = reinterpret_cast<float *>(region);
+#pragma unroll
+        for (int t = 0; t < XD_TOK; ++t) {
+            if (PAIR) {
+                f32x2 v = {a0[t], a1[t]};
+                *reinterpret_cast<f32x2 *>(bs + t * 128 + 2 * l) = v;
+            } else {
+                bs[t * 128 + l] = a0[t];
+            }
+        }
+    }
+    __syncthreads();
+    // group sums: wave w chains the block sums of tokens w and w + 8 in ascending order
+#pragma unroll
+    for (int u = 0; u < XD_TOK / XL_WAVES; ++u) {
+        const int tl = w + XL_WAVES * u;
+        const int t = t0 + tl;
+        if (t < T) {
+            if (PAIR) {
+                if (2 * l < ncols) {
+                    float s0 = 0.f, s1 = 0.f;
+                    for (int i = 0; i < nb; ++i) {
+                        const f32x2 v = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(smem + i * XL_W_BYTES) + tl * 128 + 2 * l);
+                        s0 = __fadd_rn(s0, v[0]);
+                        s1 = __fadd_rn(s1, v[1]);
+                    }
+                    f32x2 v = {s0, s1};
+                    *reinterpret_cast<f32x2 *>(sl.out + (size_t)t * sl.out_pitch + 2 * l) = v;
+                }
+            } else if (l < ncols) {
+                float s0 = 0.f;
+                for (int i = 0; i < nb; ++i) s0 = __fadd_rn(s0, reinterpret_cast<const float *>(smem + i * XL_W_BYTES)[tl * 128 + l]);
+                sl.out[(size_t)t * sl.out_pitch + l] = s0;
+            }
+        }
+    }
+}
+
 }  // namespace
 }  // namespace pto
