@@ -67,13 +67,13 @@ __host__ __device__ inline bool lip_x_group_rows(const LipParams &p)
     return p.T >= LIP_MFMA_MIN_TOKENS && !lip_x_on_matrix_cores(p) && wb >= 16 && (wb & (wb - 1)) == 0;
 }
 // partial rows [T, LIP_XCOLS] the first launch leaves per token: the blocks of 64 of the fixed-order form, or the
-// ranges of the matrix-core form (enough of them for about 256 workgroups of 128 tokens x 128 columns)
+// ranges of the matrix-core form (enough of them for about 512 workgroups of 128 tokens x 128 columns: two per compute unit)
 __host__ __device__ inline int lip_xrows(const LipParams &p)
 {
     const int nblk = p.h / LIP_XBLOCK;
     if (lip_x_group_rows(p)) return (nblk + LIP_XGROUP - 1) / LIP_XGROUP;
     if (!lip_x_on_matrix_cores(p)) return nblk;
-    int s = 128 / ((p.T + 127) / 128);
+    int s = 256 / ((p.T + 127) / 128);
     s = s < 1 ? 1 : s;
     s = s > LIP_XM_MAX_SPLITS ? LIP_XM_MAX_SPLITS : s;
     return s > nblk ? nblk : s;

@@ -71,9 +71,25 @@ static_assert(XM_KC == MLAP_XBLOCK, "the workspace is sized in chunks of the hid
 __global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams p, const int nslabs, const int nsplit)
 {
     __shared__ __attribute__((aligned(16))) uint8_t smem[XM_LDS];
-    const int slab = blockIdx.x % nslabs;
-    const int sp = (blockIdx.x / nslabs) % nsplit;
-    const int t0 = (blockIdx.x / nslabs / nsplit) * XM_TOK;
+    // Workgroups go round the eight XCDs, each with an L2 of its own, and the working set (hidden states + weights)
+    // is several times one L2: the jobs of a slab (its ranges of h x token tiles) all run on XCD slab % 8, so a slab's
+    // weights cross into one L2 only and every XCD reads the hidden states once for its two or so slabs.  The slabs
+    // left over when their number is no multiple of eight are dealt out job by job.
+    const int per_slab = nsplit * ((p.T + XM_TOK - 1) / XM_TOK);
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int full = nslabs >> 3;
+    int slab, rem;
+    if (j < full * per_slab) {
+        slab = xcd + 8 * (j / per_slab);
+        rem = j % per_slab;
+    } else {
+        const int e = (j - full * per_slab) * 8 + xcd;
+        if (e >= (nslabs & 7) * per_slab) return;      // the whole workgroup leaves, before any barrier
+        slab = 8 * full + e / per_slab;
+        rem = e % per_slab;
+    }
+    const int sp = rem % nsplit;
+    const int t0 = (rem / nsplit) * XM_TOK;
     const int qslabs = p.q_lora / 128;
     const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
     const bool isq = slab < qslabs;
@@ -304,7 +320,9 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
         ngroups = ngroups < 1 ? 1 : ngroups;
         ngroups = ngroups > MLAP_XM_MAX_SPLITS ? MLAP_XM_MAX_SPLITS : ngroups;
         ngroups = ngroups > nchunks ? nchunks : ngroups;
-        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)(nslabs * ngroups * ttiles)), dim3(256), 0, stream, p, nslabs, ngroups);
+        const int per_slab = ngroups * ttiles;
+        const int wgs = 8 * ((nslabs >> 3) * per_slab + ((nslabs & 7) * per_slab + 7) / 8);   // the kernel's XCD-wise job order
+        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p, nslabs, ngroups);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
         hipLaunchKernelGGL(mlap_xlinear_kernel, dim3((unsigned)(nslabs * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, nslabs, ngroups);
