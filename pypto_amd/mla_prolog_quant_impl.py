@@ -21,7 +21,7 @@ the last bf16 bit from the sequential statement -- inside the reference's own ac
 deepseekv32_mla_prolog_quant.py:668-692) or, when ``True``, as fixed-order fp32 sums that reproduce the
 sequential statement bit for bit.  Every other output is the same either way for fewer than 64 tokens; from 64 tokens
 on (prefill chunks) the default also takes the sums over the hidden axis (``x . w_dq``, ``x . w_dkv_kr``) on the matrix
-cores -- about thirty times faster at 512 tokens, the int8 latents then differ by one step in rare entries, inside
+cores -- sixteen times faster at 512 tokens, the int8 latents then differ by one step in rare entries, inside
 the same acceptance rule -- and ``EXACT_ABSORB = True`` keeps every sum in its fixed order.
 """
 from __future__ import annotations
