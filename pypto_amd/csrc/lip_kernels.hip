@@ -15,7 +15,7 @@
 // are balanced binary trees over neighbouring channels.  No matrix-core instruction touches these
 // sums (its internal order is not specified); only the exact integer projection uses one.
 //
-// Two launches:
+// Two launches; below LIP_MFMA_MIN_TOKENS tokens (decode):
 //   lip_linear_kernel   workgroups of four independent waves.  Two of them share a query job (head,
 //                       quarter of the reduction axis, block of 32 tokens), one half each: the tile of
 //                       w_qb (rows x 128 bytes) and the token rows travel to LDS by LDS-DMA, all
@@ -29,6 +29,16 @@
 //                       Hadamard (matrix staged in LDS once per workgroup), quantise, store.  Tokens,
 //                       one workgroup each: waves add the groups of block sums, then one wave finishes
 //                       the key row (layer norm, rope, Hadamard, quantise, scatter) and one the weights.
+// From LIP_MFMA_MIN_TOKENS tokens on (prefill chunks) the stages take forms of their own (LipParams::sum_mode says
+// which sums may leave their fixed order):
+//   lip_qproj_prefill_kernel, lip_qproj_prefill256_kernel   the query projection unsplit (prolog_common.h), a
+//                       workgroup per 128 x 128 or 256 x 256 tile over the whole reduction axis; exact.
+//   lip_xlinear_group_kernel   the fixed-order sums over the hidden axis, a group of eight blocks per workgroup and 16
+//                       tokens per weight block, hidden states broadcast by DPP (xlinear_fixed.h); or
+//   lip_xlinear_mfma_kernel    the same sums on the matrix cores (xlinear_mfma.h), if asked for.
+//   lip_finish_query_prefill_kernel   query rows with the Hadamard sums on the matrix cores, 32 rows per pass of a
+//                       wave (prolog_finish.h), unless every sum is to keep its fixed order.
+//   lip_finish_tokens_prefill_kernel  key rows and weights, eight tokens per workgroup.
 #include "lip_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"

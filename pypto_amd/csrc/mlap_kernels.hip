@@ -8,17 +8,15 @@
 // has a fixed order (all products are bf16 x bf16, exact in fp32): sums over the hidden axis in blocks of
 // 64 ascending, eight block sums ascending into a group sum, group sums ascending; the RMS sums as a
 // balanced tree over the 128 channels of a slab, slab sums ascending; the 128-term sums against w_uk
-// ascending.  Only the exact integer projection runs on the matrix cores.
+// ascending.  In that form only the exact integer projection runs on the matrix cores; the caller may let the
+// sums against w_uk, and from MLAP_MFMA_MIN_TOKENS tokens on the sums over the hidden axis, run there as well
+// (MlapParams::absorb_exact = 0: the same exact products in the cores' own summation order).
 //
-// Four launches:
-//   mlap_xlinear_kernel  x . [w_dq | w_dkv_kr]: one workgroup of eight waves per (slab of 128 columns,
-//                        group of 512 hidden rows, 8 tokens); each wave takes a 64-row block (staged by
+// Four launches; below MLAP_MFMA_MIN_TOKENS tokens (decode):
+//   mlap_xlinear_kernel  x . [w_dq | w_dkv_kr] (xlinear_fixed.h): one workgroup of eight waves per (slab of 128
+//                        columns, group of 512 hidden rows, 8 tokens); each wave takes a 64-row block (staged by
 //                        LDS-DMA, hidden states widened to fp32 in LDS), block sums meet in LDS and are
 //                        chained into the group sum.
-//   mlap_xlinear_mfma_kernel  the same sums on the matrix cores, taken from MLAP_MFMA_MIN_TOKENS tokens
-//                        on unless the fixed order is asked for: per workgroup a 128-column slab x 128
-//                        tokens x a quarter of the hidden axis, v_mfma_f32_32x32x16_bf16 with the
-//                        row-major weight chunk as the transposed operand (ds_read_b64_tr_b16).
 //   mlap_mid_kernel      per token: group sums chained, bf16, RMS norm (one wave per slab), per-token
 //                        int8 quantisation of the query latent; RMS norm and per-slab quantisation of
 //                        the key latent, rope of the key, scatter into the caches.
@@ -26,7 +24,15 @@
 //                        v_perm_b32 transposes, v_mfma_i32_32x32x32_i8), partial sums per quarter.
 //   mlap_finish_kernel   per (head, half of the 512 output columns, 8 tokens): partial sums added and
 //                        de-quantised, rope part rotated and stored, nope part times the head's w_uk
-//                        slice (staged in LDS by LDS-DMA), one output column per lane, 8 tokens at once.
+//                        slice (staged in LDS by LDS-DMA): on the matrix cores, or one output column per lane.
+// From MLAP_MFMA_MIN_TOKENS tokens on (prefill chunks) the stages take forms of their own:
+//   mlap_xlinear_mfma_kernel   the sums over the hidden axis on the matrix cores (xlinear_mfma.h) unless the fixed
+//                        order is asked for: per workgroup a 128-column slab x 128 tokens x a range of the hidden
+//                        axis, v_mfma_f32_32x32x16_bf16 with the row-major weight chunk as the transposed operand.
+//   qproj_prefill_kernel, qproj_prefill256_kernel   the projection unsplit (prolog_common.h), a workgroup per
+//                        128 x 128 or 256 x 256 tile over the whole reduction axis; results leave de-quantised.
+//   mlap_finish_prefill_kernel   per (head, run of 32-token blocks): the head's whole w_uk staged once
+//                        (prolog_finish.h), absorb product on the matrix cores.
 #include "mlap_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"
