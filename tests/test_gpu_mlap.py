@@ -193,8 +193,8 @@ def run_fused(dm, dl, t, n, n_idx, op=None):
     return q_nope, q_rope, q_int8, q_scale, weights
 
 
-@pytest.mark.parametrize("mode", ["default", "exact", "matrix_cores"])
-def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode):
+@pytest.mark.parametrize("mode,shape", [("default", "small"), ("exact", "small"), ("matrix_cores", "small"), ("default", "t_512")])
+def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, shape):
     """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
     projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
     indexer prolog called one after the other on the same inputs, bit for bit, in each of the summation modes."""
@@ -203,11 +203,15 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode):
     from pypto_amd.synthetic import gen_indexer_prolog_inputs
     impl.EXACT_ABSORB = lip_impl.EXACT_SUMS = mode == "exact"
     lip_impl.MATRIX_CORE_HIDDEN_SUMS = mode == "matrix_cores"
-    kw = dict(h=256, q_lora_rank=512)
-    b, s1, act = 3, 50, [700, 650, 600]
+    if shape == "small":
+        kw = dict(h=256, q_lora_rank=512)
+        b, s1, act, n_mla, n_idx = 3, 50, [700, 650, 600], 4, 8
+    else:   # the reference's test_t_512_tilebs_128_p (deepseekv32_mla_indexer_prolog_quant.py:1050-1117) at the model's sizes
+        kw = {}
+        b, s1, act, n_mla, n_idx = 128, 4, [4096] * 128, 128, 64
     dev = torch.device("cuda:0")
-    mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=4, **kw)
-    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=8, **kw)
+    mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=n_mla, **kw)
+    lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=n_idx, **kw)
     t = b * s1
     # separate operators
     sep = run_op(mla, (1e-5, 1e-5), prefill=True)
@@ -216,14 +220,14 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode):
     dm0 = mla.to(dev)
     la[0], la[1], la[2] = dm0.token_x, torch.from_numpy(sep["q_norm"]).to(dev), torch.from_numpy(sep["q_norm_scale"]).reshape(-1, 1).to(dev)
     la[9], la[10], la[15] = dm0.cos, dm0.sin, dm0.cache_index
-    s_q = torch.empty([t, 8, 128], dtype=torch.int8, device=dev)
-    s_sc = torch.empty([t, 8, 1], dtype=torch.float16, device=dev)
-    s_w = torch.empty([t, 8], dtype=torch.float16, device=dev)
+    s_q = torch.empty([t, n_idx, 128], dtype=torch.int8, device=dev)
+    s_sc = torch.empty([t, n_idx, 1], dtype=torch.float16, device=dev)
+    s_w = torch.empty([t, n_idx], dtype=torch.float16, device=dev)
     pypto_amd.lightning_indexer_prolog_quant(*la, s_q, s_sc, dl.k_cache, dl.k_cache_scale, s_w)
     torch.cuda.synchronize()
     # fused
     dm, dl2 = mla.to(dev), lip.to(dev)
-    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl2, t, 4, 8, op=pypto_amd.mla_indexer_prolog_quant_p)
+    q_nope, q_rope, q_int8, q_scale, weights = run_fused(dm, dl2, t, n_mla, n_idx, op=pypto_amd.mla_indexer_prolog_quant_p)
     assert np.array_equal(q_nope.float().cpu().numpy(), sep["query_nope"])
     assert np.array_equal(q_rope.float().cpu().numpy(), sep["query_rope"])
     assert np.array_equal(dm.kv_cache.cpu().numpy(), sep["kv_cache"])
