@@ -312,10 +312,12 @@ def prefill_prologs_leg(torch, pypto_amd, dev):
     from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
 
-    def timed(fn, n=10):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
+    def timed(fn, n=20):
+        t_settle = time.perf_counter()                  # 0.3 s of untimed calls: the device clocks rise under load
+        while time.perf_counter() - t_settle < 0.3:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(n):
