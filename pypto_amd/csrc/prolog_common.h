@@ -206,10 +206,37 @@ __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const 
     }
 }
 
+// Weight operands for the unsplit forms by the transposing 8-bit LDS read.  ds_read_b64_tr_b8 takes, per group of
+// 16 lanes, the 16 rows of 8 bytes its lanes point at and hands lane j byte j of the even lanes' rows and lane 8 + j
+// byte j of the odd lanes' rows.  Even lanes point at eight consecutive rows of the tile at one block of 8 columns,
+// odd lanes at the same rows of the next block: lane n of the group then holds column n of 16, eight rows deep --
+// half of what v_mfma_i32_32x32x32_i8 wants from a lane (column l % 32, rows 16*(l / 32) .. +15), so two reads per
+// product and no byte shuffling.  Product i covers columns 32*i .. 32*i + 31 of the slab.
+// Tile layout the reads assume: row r (128 bytes) keeps its 16-byte piece q at piece q ^ 2*((r >> 1) & 3), so that
+// the eight rows of a half-wave's read fall on different banks; the LDS-DMA requests place the pieces that way.
+__device__ __forceinline__ int q_tr_piece_swizzle(const int row) { return 2 * ((row >> 1) & 3); }
+
+__device__ __forceinline__ void q_build_a_tr(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
+{
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    const int x = (l >> 2) & 3;                         // (row >> 1) & 3 of this lane's rows
+    const uint8_t *base = tile + (32 * s + 16 * (l >> 5) + ((l & 15) >> 1)) * 128 + 16 * ((l >> 4) & 1) + 8 * (l & 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint8_t *pi = base + 32 * (i ^ x);
+        const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)pi);
+        const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)(pi + 8 * 128));
+        a[i][0] = lo[0];
+        a[i][1] = lo[1];
+        a[i][2] = hi[0];
+        a[i][3] = hi[1];
+    }
+}
+
 // The unsplit forms' results leave de-quantised, as bf16, through a staging area of the wave's own in LDS
 // (Q_STAGE_BYTES; the chunk buffers are free by then), so that they reach memory as whole 256-byte rows instead of
-// 8-byte fragments of 32 different rows: accumulator register r of the four products holds columns 4m .. 4m+3 of this
-// lane's token (m as in q_pair_store_from).  tbase: first of the wave's 32 tokens; col0: first of its 128 columns.
+// 8-byte fragments of 32 different rows: registers 4*rg .. 4*rg+3 of product i hold columns 32*i + 8*rg + 4*(l/32) .. +3
+// of this lane's token (q_build_a_tr).  tbase: first of the wave's 32 tokens; col0: first of its 128 columns.
 constexpr int Q_STAGE_PITCH = 272;                     // bytes between token rows: 16-byte aligned, 4 banks apart
 constexpr int Q_STAGE_BYTES = 32 * Q_STAGE_PITCH;
 __device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16 (&acc)[4], const int tbase, const int col0, const int l,
@@ -221,15 +248,17 @@ __device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16
     const float *cs = p.col_scale + col0;
     uint8_t *mine = stage + (l & 31) * Q_STAGE_PITCH;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
-        const f32x4 c = *reinterpret_cast<const f32x4 *>(cs + 4 * m);
-        float v[4];
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = __fmul_rn(__fmul_rn((float)acc[i][r], ts), c[i]);
-        const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-        *reinterpret_cast<u32x2 *>(mine + 8 * m) = o;
-    }
+        for (int rg = 0; rg < 4; ++rg) {
+            const int col = 32 * i + 8 * rg + 4 * (l >> 5);
+            const f32x4 c = *reinterpret_cast<const f32x4 *>(cs + col);
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = __fmul_rn(__fmul_rn((float)acc[i][4 * rg + j], ts), c[j]);
+            const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<u32x2 *>(mine + 2 * col) = o;
+        }
     // the wave reads back what it wrote itself: LDS operations of a wave stay in order
     uint16_t *dst = reinterpret_cast<uint16_t *>(p.part) + col0 + 8 * (l & 15);
 #pragma unroll
@@ -245,7 +274,8 @@ __device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16
 // columns, block of 128 tokens) walks the whole reduction axis in chunks of 128 rows, so a weight tile is read
 // once per 128 tokens instead of once per 32 and no partial sums are left to add.  Wave w takes tokens 32w..32w+31
 // of the block; the chunk of the tile (16 KiB, shared) and each wave's token operands (4 KiB) travel by LDS-DMA into
-// one of two buffers, a chunk ahead of the products that read them.  Same products and lane layout as a split job.
+// one of two buffers, a chunk ahead of the products that read them.  Same products as a split job; the weight
+// operands come out of LDS by the transposing 8-bit read (q_build_a_tr) instead of byte shuffles.
 constexpr int QPF_STEPS = 4;                           // 32-row steps per chunk
 constexpr int QPF_TILE = QPF_STEPS * 32 * 128;
 constexpr int QPF_TOK = QPF_STEPS * 1024;
@@ -265,15 +295,15 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
     const int t = (job % ttiles) * 128 + 32 * w + (l & 31);
     const int nch = p.q_lora / (32 * QPF_STEPS);
     const int8_t *tsrc = p.q_norm + (size_t)(t < p.T ? t : p.T - 1) * p.q_lora + 16 * (l >> 5);
-    const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * (l & 7);
-    const int8_t *wswp = p.w + (size_t)(32 * w + ((l >> 3) ^ 1)) * ncols + slab * 128 + 16 * (l & 7);   // rows 16..31 of a step: neighbours swapped
+    // lane l of a tile request fills piece l % 8 of row l / 8 of its eight rows: with the piece that belongs there (q_build_a_tr)
+    const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * ((l & 7) ^ q_tr_piece_swizzle(l >> 3));
     const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
     auto issue = [&](const int c) {
         const uint32_t buf = base + (c & 1) * QPF_BUF;
 #pragma unroll
         for (int s = 0; s < QPF_STEPS; ++s) dma16(tsrc + c * (32 * QPF_STEPS) + 32 * s, buf + QPF_TILE + w * QPF_TOK + 1024 * s);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16((i < 2 ? wsrc : wswp) + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
+        for (int i = 0; i < 4; ++i) dma16(wsrc + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
     };
     i32x16 acc[4];
 #pragma unroll
@@ -292,7 +322,13 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
         __syncthreads();                               // every wave's share of chunk c has landed
         const uint8_t *buf = lds + (c & 1) * QPF_BUF;
 #pragma unroll
-        for (int s = 0; s < QPF_STEPS; ++s) q_step_at(buf, buf + QPF_TILE + w * QPF_TOK, s, l, acc);
+        for (int s = 0; s < QPF_STEPS; ++s) {
+            i32x4 a[4];
+            q_build_a_tr(buf, s, l, a);
+            const i32x4 b = *reinterpret_cast<const i32x4 *>(buf + QPF_TILE + w * QPF_TOK + 1024 * s + 16 * l);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+        }
         __syncthreads();                               // chunk c + 2 goes where chunk c was read
     }
     static_assert(4 * Q_STAGE_BYTES <= QPF_LDS, "the staging areas reuse the chunk buffers");
@@ -323,7 +359,7 @@ __device__ __forceinline__ void q_prefill256_body(const QProj &p, const int job,
     const bool cols_live = 2 * ct + wc < p.nslabs;      // an odd number of slabs leaves the last tile half empty
     const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
     // this wave's four requests of a chunk: tile pieces 2w, 2w+1 (half = piece / 8; rows 8*(piece % 8) .. +7 of the
-    // chunk, neighbours swapped in rows 16..31 of a step) and token pieces 2w, 2w+1 (token block w, steps 0 and 1)
+    // chunk, 16-byte pieces placed as q_build_a_tr reads them) and token pieces 2w, 2w+1 (token block w, steps 0 and 1)
     const int8_t *tsrc[2];
     uint32_t tdst[2];
 #pragma unroll
@@ -331,8 +367,7 @@ __device__ __forceinline__ void q_prefill256_body(const QProj &p, const int job,
         const int q = 2 * w + j;
         const int half = q >> 3, rb = q & 7;
         const int slab = 2 * ct + half < p.nslabs ? 2 * ct + half : p.nslabs - 1;
-        const int row = 8 * rb + (((rb & 3) >= 2) ? ((l >> 3) ^ 1) : (l >> 3));
-        tsrc[j] = p.w + (size_t)row * ncols + slab * 128 + 16 * (l & 7);
+        tsrc[j] = p.w + (size_t)(8 * rb + (l >> 3)) * ncols + slab * 128 + 16 * ((l & 7) ^ q_tr_piece_swizzle(l >> 3));
         tdst[j] = half * 8192 + rb * 1024;
     }
     int t = t0 + 32 * w + (l & 31);
@@ -366,7 +401,7 @@ __device__ __forceinline__ void q_prefill256_body(const QProj &p, const int job,
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 i32x4 a[4];
-                q_build_a(bp + wc * 8192, s, l, a);
+                q_build_a_tr(bp + wc * 8192, s, l, a);
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb) {
                     const i32x4 b = *reinterpret_cast<const i32x4 *>(bp + 16384 + (2 * (2 * wt + tb) + s) * 1024 + 16 * l);
