@@ -48,28 +48,29 @@ __device__ __forceinline__ void xm_body(const XmSlab &sl, const uint16_t *x, con
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_byte_t *)smem;
 
     // this wave's eight requests of a chunk: four of the slab (four rows each), four of the hidden states (eight
-    // token rows each)
+    // token rows each).  Their addresses are made once, for chunk 0; a chunk further on is a uniform number of bytes
+    // further on (the loop then spends two additions per request instead of rebuilding the addresses).
     const int wrow = l >> 4, wpos = l & 15;
     const uint32_t woff = (uint32_t)(wrow * sl.pitch + 16 * (narrow ? (wpos < sl.pieces ? wpos : 0) : (wpos ^ (4 * wrow))));
     const uint64_t wmask = narrow ? ((1ull << sl.pieces) - 1) * 0x0001000100010001ull : ~0ull;
     const int xrow = l >> 3, xpos = l & 7;
+    const uint8_t *wreq[4], *xreq[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int req = 4 * w + j;
+        wreq[j] = sl.w + (size_t)(4 * req) * sl.pitch + woff;
+        const int tl = 8 * req + xrow;                              // token row inside the workgroup's 128
+        int t = t0 + tl;
+        t = t < T ? t : T - 1;
+        xreq[j] = reinterpret_cast<const uint8_t *>(x) + (size_t)t * h * 2 + 16 * (xpos ^ ((tl >> 1) & 7));
+    }
+    const size_t wstep = (size_t)XM_KC * sl.pitch;
     auto request_chunk = [&](const int c, const int buf) {
         const uint32_t dst = lds0 + (uint32_t)(buf * XM_BUF);
-        const uint8_t *wsrc = sl.w + (size_t)(c * XM_KC) * sl.pitch + woff;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int req = 4 * w + j;
-            dma16_lanes(wsrc + (size_t)(4 * req) * sl.pitch, dst + 1024u * req, wmask);
-        }
+        for (int j = 0; j < 4; ++j) dma16_lanes(wreq[j] + (size_t)c * wstep, dst + 1024u * (4 * w + j), wmask);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int req = 4 * w + j;
-            const int tl = 8 * req + xrow;                          // token row inside the workgroup's 128
-            int t = t0 + tl;
-            t = t < T ? t : T - 1;
-            dma16(reinterpret_cast<const uint8_t *>(x) + ((size_t)t * h + (size_t)c * XM_KC) * 2 + 16 * (xpos ^ ((tl >> 1) & 7)),
-                  dst + XM_W_BYTES + 1024u * req);
-        }
+        for (int j = 0; j < 4; ++j) dma16(xreq[j] + (size_t)c * (XM_KC * 2), dst + XM_W_BYTES + 1024u * (4 * w + j));
     };
 
     f32x16 acc[2][2];
