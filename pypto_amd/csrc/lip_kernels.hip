@@ -311,12 +311,13 @@ hipError_t lip_launch_finish(const LipParams &p, hipStream_t stream)
 {
     const int q_wgs = lip_finish_query_wgs(p);
     if (lip_q_on_matrix_cores(p)) {
-        // the query rows on the matrix cores, in passes of 32 rows per wave, at most two workgroups per compute unit
+        // the query rows on the matrix cores, in passes of 32 rows per wave, as many workgroups as are resident at once
         const int npass = (p.T * p.n_heads + 31) / 32;
         const int cus = cu_count();
         if (cus <= 0) return hipErrorNoDevice;
         int wgs = (npass + QFP_WAVES - 1) / QFP_WAVES;
-        wgs = wgs > 2 * cus ? 2 * cus : wgs;
+        const int resident = cus * (160 * 1024 / LIP_QFP_LDS);
+        wgs = wgs > resident ? resident : wgs;
         hipLaunchKernelGGL(lip_finish_query_prefill_kernel, dim3((unsigned)wgs), dim3(64 * QFP_WAVES), 0, stream, p);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

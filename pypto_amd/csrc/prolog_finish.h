@@ -343,6 +343,7 @@ constexpr int QFP_OPITCH = 144;                        // bytes between int8 row
 constexpr int QFP_WAVE_BYTES = 32 * QFP_APITCH * 2;
 constexpr int LIP_QFP_LDS = LIP_DIM * QFP_HPITCH * 2 + QFP_WAVES * QFP_WAVE_BYTES;   // 69 632 bytes
 static_assert(32 * QFP_OPITCH <= QFP_WAVE_BYTES, "the int8 rows reuse the operand buffer");
+static_assert(LIP_QFP_LDS <= 160 * 1024, "one workgroup fits a compute unit");
 
 __device__ __forceinline__ void lip_finish_query_prefill_body(const LipParams &p, const int wg, const int nwg, uint8_t *lds)
 {
@@ -362,30 +363,45 @@ __device__ __forceinline__ void lip_finish_query_prefill_body(const LipParams &p
     const int npass = (nrows + 31) / 32;
     const uint16_t *at = abf + (l & 31) * QFP_APITCH + 4 * (l >> 5);
     const uint16_t *wt = hmat + (4 * (l >> 5) + ((l & 15) >> 2)) * QFP_HPITCH + 16 * ((l >> 4) & 1) + 4 * (l & 3);
-#pragma unroll 1
-    for (int pass = wg * QFP_WAVES + w; pass < npass; pass += nwg * QFP_WAVES) {
-#pragma unroll 1
-        for (int b8 = 0; b8 < 4; ++b8) {
-            uint32_t raw[8];
-            uint32_t rc[8], rs[8];
+    // Eight rows at a time; the loads of the next eight (of this pass or of the wave's next one) are on their way
+    // while the current eight are rotated: a pass would otherwise wait out four memory round trips.
+    struct Rows8 {
+        uint32_t raw[8], rc[8], rs[8];
+    };
+    auto load_rows = [&](Rows8 &r, const int pass, const int b8) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int row = pass * 32 + b8 * 8 + u;
-                const int rr = row < nrows ? row : nrows - 1;
-                const int t = rr / p.n_heads;
-                const int col = (rr - t * p.n_heads) * LIP_DIM + 2 * l;
-                raw[u] = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(p.qpart) + (size_t)t * ncols + col);
-                rc[u] = rope_coef(p.cos, t, l);
-                rs[u] = rope_coef(p.sin, t, l);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                float v0 = __uint_as_float(raw[u] << 16);      // the unsplit projection leaves its results de-quantised
-                float v1 = __uint_as_float(raw[u] & 0xffff0000u);
-                rope_pair(v0, v1, rc[u], rs[u], l);
-                *reinterpret_cast<uint32_t *>(abf + (b8 * 8 + u) * QFP_APITCH + 2 * l) = pack_bf16x2(v0, v1);
-            }
+        for (int u = 0; u < 8; ++u) {
+            const int row = pass * 32 + b8 * 8 + u;
+            const int rr = row < nrows ? row : nrows - 1;
+            const int t = rr / p.n_heads;
+            const int col = (rr - t * p.n_heads) * LIP_DIM + 2 * l;
+            r.raw[u] = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(p.qpart) + (size_t)t * ncols + col);
+            r.rc[u] = rope_coef(p.cos, t, l);
+            r.rs[u] = rope_coef(p.sin, t, l);
         }
+    };
+    auto rotate_rows = [&](const Rows8 &r, const int b8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            float v0 = __uint_as_float(r.raw[u] << 16);        // the unsplit projection leaves its results de-quantised
+            float v1 = __uint_as_float(r.raw[u] & 0xffff0000u);
+            rope_pair(v0, v1, r.rc[u], r.rs[u], l);
+            *reinterpret_cast<uint32_t *>(abf + (b8 * 8 + u) * QFP_APITCH + 2 * l) = pack_bf16x2(v0, v1);
+        }
+    };
+    const int stride = nwg * QFP_WAVES;
+    Rows8 ra, rb;
+    if (wg * QFP_WAVES + w < npass) load_rows(ra, wg * QFP_WAVES + w, 0);
+#pragma unroll 1
+    for (int pass = wg * QFP_WAVES + w; pass < npass; pass += stride) {
+        load_rows(rb, pass, 1);
+        rotate_rows(ra, 0);
+        load_rows(ra, pass, 2);
+        rotate_rows(rb, 1);
+        load_rows(rb, pass, 3);
+        rotate_rows(ra, 2);
+        if (pass + stride < npass) load_rows(ra, pass + stride, 0);
+        rotate_rows(rb, 3);
         // the wave reads back what it wrote itself: LDS operations of a wave stay in order
         f32x16 c[4];
 #pragma unroll
