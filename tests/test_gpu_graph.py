@@ -61,15 +61,16 @@ def test_indexer_then_attention_replays_match_eager():
         assert torch.equal(got.view(torch.int16), out_e.view(torch.int16)), f"replay {rep}: attention differs"
 
 
-def test_prologs_replays_match_eager():
-    """MLA prolog + indexer prolog (the fused operator) recorded once; hidden states change in place between
-    replays, the caches start from the same state each time."""
+@pytest.mark.parametrize("b,s1,act,ni", [(4, 2, [5000, 300, 129, 64], 4),      # decode kernels
+                                         (3, 50, [700, 650, 600], 8)])         # 150 tokens: the prefill forms of every stage
+def test_prologs_replays_match_eager(b, s1, act, ni):
+    """MLA prolog + indexer prolog recorded once; hidden states change in place between replays, the caches start
+    from the same state each time."""
     from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
     dev = torch.device(DEV)
-    b, s1, act = 4, 2, [5000, 300, 129, 64]
     kw = dict(h=512, q_lora_rank=1536)
     mla = gen_mla_prolog_inputs(b, s1, act, seed=21, n_heads=8, **kw).to(dev)
-    lip = gen_indexer_prolog_inputs(b, s1, act, seed=22, n_heads=4, **kw).to(dev)
+    lip = gen_indexer_prolog_inputs(b, s1, act, seed=22, n_heads=ni, **kw).to(dev)
     t = b * s1
     caches = [mla.kv_cache, mla.kr_cache, mla.k_scale_cache, lip.k_cache, lip.k_cache_scale]
     base = [c.clone() for c in caches]
@@ -77,8 +78,8 @@ def test_prologs_replays_match_eager():
     def outputs():
         return (torch.zeros(t, 1536, dtype=torch.int8, device=dev), torch.zeros(t, 1, device=dev),
                 torch.zeros(t, 8, 512, dtype=torch.bfloat16, device=dev), torch.zeros(t, 8, 64, dtype=torch.bfloat16, device=dev),
-                torch.zeros(t, 4, 128, dtype=torch.int8, device=dev), torch.zeros(t, 4, 1, dtype=torch.float16, device=dev),
-                torch.zeros(t, 4, dtype=torch.float16, device=dev))
+                torch.zeros(t, ni, 128, dtype=torch.int8, device=dev), torch.zeros(t, ni, 1, dtype=torch.float16, device=dev),
+                torch.zeros(t, ni, dtype=torch.float16, device=dev))
 
     def run(o):
         qn, qs, qnope, qrope, iq, iqs, iw = o
