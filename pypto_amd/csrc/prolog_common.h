@@ -294,14 +294,23 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
     const int slab = job / ttiles;
     const int t = (job % ttiles) * 128 + 32 * w + (l & 31);
     const int nch = p.q_lora / (32 * QPF_STEPS);
-    const int8_t *tsrc = p.q_norm + (size_t)(t < p.T ? t : p.T - 1) * p.q_lora + 16 * (l >> 5);
+    // token operands: a request brings 128 bytes (the chunk's four steps) of 8 tokens -- whole lines; as 32 tokens x 32
+    // bytes a request runs at half the rate.  Lane l fills piece l % 8 of token row l / 8 with piece (l % 8) ^ (l / 8)
+    // of that token, so that the operand reads of 8 consecutive tokens fall on different banks.
+    const int8_t *tsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int tq = (job % ttiles) * 128 + 32 * w + 8 * i + (l >> 3);
+        tq = tq < p.T ? tq : p.T - 1;                  // rows past the end repeat the last token and are not stored
+        tsrc[i] = p.q_norm + (size_t)tq * p.q_lora + 16 * ((l & 7) ^ (l >> 3));
+    }
     // lane l of a tile request fills piece l % 8 of row l / 8 of its eight rows: with the piece that belongs there (q_build_a_tr)
     const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * ((l & 7) ^ q_tr_piece_swizzle(l >> 3));
     const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
     auto issue = [&](const int c) {
         const uint32_t buf = base + (c & 1) * QPF_BUF;
 #pragma unroll
-        for (int s = 0; s < QPF_STEPS; ++s) dma16(tsrc + c * (32 * QPF_STEPS) + 32 * s, buf + QPF_TILE + w * QPF_TOK + 1024 * s);
+        for (int i = 0; i < 4; ++i) dma16(tsrc[i] + c * (32 * QPF_STEPS), buf + QPF_TILE + w * QPF_TOK + 1024 * i);
 #pragma unroll
         for (int i = 0; i < 4; ++i) dma16(wsrc + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
     };
@@ -325,7 +334,7 @@ __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, ui
         for (int s = 0; s < QPF_STEPS; ++s) {
             i32x4 a[4];
             q_build_a_tr(buf, s, l, a);
-            const i32x4 b = *reinterpret_cast<const i32x4 *>(buf + QPF_TILE + w * QPF_TOK + 1024 * s + 16 * l);
+            const i32x4 b = *reinterpret_cast<const i32x4 *>(buf + QPF_TILE + w * QPF_TOK + (l & 31) * 128 + 16 * ((2 * s + (l >> 5)) ^ (l & 7)));
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
         }
