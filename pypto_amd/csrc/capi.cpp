@@ -331,7 +331,7 @@ extern "C" {
 
 const char *pto_last_error(void) { return g_err; }
 
-const char *pto_version(void) { return "0.5.0"; }
+const char *pto_version(void) { return "0.5.1"; }
 
 int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
 {
@@ -556,6 +556,7 @@ static int lip_params(const PtoLiPrologQuantArgs *a, pto::LipParams &p)
     p.n_heads = (int)a->n_heads;
     p.eps = a->eps;
     p.sum_mode = a->sum_mode;
+    p.x_in_groups = 0;
     p.w_mul0 = (float)std::pow((double)a->n_heads, -0.5);
     p.w_mul1 = (float)std::pow((double)pto::LIP_DIM, -0.5);
     return PTO_OK;

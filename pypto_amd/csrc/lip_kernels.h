@@ -41,6 +41,8 @@ struct LipParams {
     int T, h, q_lora, n_heads;
     float eps, w_mul0, w_mul1;   // weights = fp16((bf16(x.w_proj) * w_mul0) * w_mul1)
     int sum_mode;                // LIP_SUMS_*
+    int x_in_groups;             // 1: xpart already holds one row per group of eight blocks, left there by another
+                                 // operator's launch (the fused prolog at decode sizes); set by that launcher only
 };
 
 // How the fp32 sums are taken from LIP_MFMA_MIN_TOKENS tokens on (below that every sum has its fixed order):
@@ -64,6 +66,7 @@ __host__ __device__ inline bool lip_x_on_matrix_cores(const LipParams &p)
 __host__ __device__ inline bool lip_x_group_rows(const LipParams &p)
 {
     const int wb = p.n_heads * 2;
+    if (p.x_in_groups) return true;
     return p.T >= LIP_MFMA_MIN_TOKENS && !lip_x_on_matrix_cores(p) && wb >= 16 && (wb & (wb - 1)) == 0;
 }
 // partial rows [T, LIP_XCOLS] the first launch leaves per token: the blocks of 64 of the fixed-order form, or the

@@ -58,9 +58,25 @@ struct MlapParams {
                                   // MLAP_MFMA_MIN_TOKENS tokens on the sums over the hidden axis as well
 };
 
+// Work of the lightning-indexer prolog that the decode form's launches can carry along (the fused operator): its
+// sums over the hidden axis have the same fixed order as this prolog's and its int8 projection reads the same
+// q_norm, so wk rides as one more column slab of the first launch, w_proj shares the slab of w_dkv_kr's 64 rope
+// columns, and the projection's jobs follow this prolog's in the third launch.
+struct MlapRider {
+    const uint16_t *wk;      // [h, 128] bf16
+    const uint16_t *w_proj;  // [h, 64] bf16
+    float *xpart;            // group sums [ceil(h/512), T, 192]: wk's columns, then w_proj's
+    const int8_t *w_qb;      // [q_lora, 128 * q_slabs] int8
+    int32_t *qpart;          // partial sums [4, T, 128 * q_slabs]
+    int q_slabs;
+};
+
+// whether the launches of `p` take a rider at all: the decode form only
+inline bool mlap_takes_rider(const MlapParams &p) { return p.T < MLAP_MFMA_MIN_TOKENS; }
+
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
 // all launches but the last, and the number of workgroups of the last (for the fused operator's last launch)
-hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream);
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider = nullptr);
 int mlap_finish_wgs(const MlapParams &p);
 // the last launch alone; at prefill sizes (mlap_finish_is_prefill) it has a form of its own that the fused operator
 // launches beside, not inside, its own last launch

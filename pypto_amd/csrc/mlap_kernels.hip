@@ -25,6 +25,8 @@
 //   mlap_finish_kernel   per (head, half of the 512 output columns, 8 tokens): partial sums added and
 //                        de-quantised, rope part rotated and stored, nope part times the head's w_uk
 //                        slice (staged in LDS by LDS-DMA): on the matrix cores, or one output column per lane.
+// For the fused operator the first and the third of these carry the lightning-indexer prolog's first stage along
+// (MlapRider in mlap_kernels.h: its hidden-axis sums have this prolog's fixed order, its projection this one's q_norm).
 // From MLAP_MFMA_MIN_TOKENS tokens on (prefill chunks) the stages take forms of their own:
 //   mlap_xlinear_mfma_kernel   the sums over the hidden axis on the matrix cores (xlinear_mfma.h) unless the fixed
 //                        order is asked for: per workgroup a 128-column slab x 128 tokens x a range of the hidden
@@ -47,10 +49,12 @@ namespace {
 static_assert(QPROJ_KSPLIT == QPROJ_KSPLIT_HOST, "workspace sizing and kernels disagree");
 
 static_assert(XL_BLOCK == MLAP_XBLOCK && XL_GROUP == MLAP_XGROUP && XL_TOK == MLAP_XTOK, "workspace sizing and kernels disagree");
+constexpr int RIDER_XCOLS = 192;     // columns of a row of the rider's group sums: wk's 128, then w_proj's 64
 
 // Fixed-order sums over the hidden axis (xlinear_fixed.h).  Column slabs: 0 .. q_lora/128 - 1 of w_dq, then four
 // slabs of w_dkv_kr's latent part and one half slab (64 columns) of its rope part.
-__global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapParams p, const int nslabs, const int ngroups)
+// With a rider (mlap_kernels.h) there is one slab more, wk's 128 columns, and the rope slab's upper half is w_proj.
+__global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapParams p, const int nslabs, const int ngroups, const MlapRider rd)
 {
     __shared__ __attribute__((aligned(16))) uint8_t smem[XL_LDS];
     const int slab = blockIdx.x % nslabs;
@@ -60,11 +64,26 @@ __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapP
     const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
     const bool isq = slab < qslabs;
     XlSlab sl;
-    sl.w = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256 : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
-    sl.pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
-    sl.wbytes = (!isq && slab - qslabs == 4) ? 128 : 256;
-    sl.out = p.xpart + (size_t)g * p.T * nc + slab * 128;
-    sl.out_pitch = nc;
+    if (slab == qslabs + 5) {
+        sl.w = reinterpret_cast<const uint8_t *>(rd.wk);
+        sl.pitch = 256;
+        sl.wbytes = 256;
+        sl.out = rd.xpart + (size_t)g * p.T * RIDER_XCOLS;
+        sl.out_pitch = RIDER_XCOLS;
+    } else {
+        sl.w = isq ? reinterpret_cast<const uint8_t *>(p.w_dq) + slab * 256 : reinterpret_cast<const uint8_t *>(p.w_dkvkr) + (slab - qslabs) * 256;
+        sl.pitch = (isq ? p.q_lora : MLAP_KV + MLAP_ROPE) * 2;
+        sl.wbytes = (!isq && slab - qslabs == 4) ? 128 : 256;
+        sl.out = p.xpart + (size_t)g * p.T * nc + slab * 128;
+        sl.out_pitch = nc;
+        if (sl.wbytes == 128 && rd.w_proj != nullptr) {
+            sl.wbytes = 256;
+            sl.w_hi = reinterpret_cast<const uint8_t *>(rd.w_proj);
+            sl.pitch_hi = 128;
+            sl.out_hi = rd.xpart + (size_t)g * p.T * RIDER_XCOLS + 128;
+            sl.out_pitch_hi = RIDER_XCOLS;
+        }
+    }
     xl_body(sl, p.x, p.T, p.h, g, t0, smem);
 }
 
@@ -228,8 +247,9 @@ constexpr int qproj_lds_bytes()
     return 4 * HS * (32 * 128 + 1024) + 2 * LIN_RED_BYTES;
 }
 
+// Jobs [0, njobs_a) belong to projection pa, jobs [njobs_a, njobs) to pb (same q_norm and reduction axis: the rider's).
 template <int HS>
-__global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njobs)
+__global__ __launch_bounds__(128) void qproj_kernel(const QProj pa, const int njobs_a, const QProj pb, const int njobs)
 {
     constexpr int BUF = HS * (32 * 128 + 1024);
     constexpr int NREQ = HS * 5;                       // requests of one job per wave
@@ -239,11 +259,15 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njo
     uint8_t *bufs = smem + w * 2 * BUF;
     uint8_t *park = smem + 4 * BUF;
     int job = blockIdx.x;
-    if (job < njobs) q_issue<HS>(p, bufs, job, w);
+    const auto issue = [&](uint8_t *region, const int j) {
+        if (j < njobs_a) q_issue<HS>(pa, region, j, w);
+        else q_issue<HS>(pb, region, j - njobs_a, w);
+    };
+    if (job < njobs) issue(bufs, job);
     for (int k = 0; job < njobs; job += gridDim.x, ++k) {
         const int next = job + gridDim.x;
         if (next < njobs) {
-            q_issue<HS>(p, bufs + ((k + 1) & 1) * BUF, next, w);
+            issue(bufs + ((k + 1) & 1) * BUF, next);
             VM_WAIT(NREQ);
         } else {
             VM_WAIT(0);
@@ -259,7 +283,10 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj p, const int njo
         uint8_t *pk = park + (k & 1) * LIN_RED_BYTES;
         if (w == 1) q_pair_park(pk, l, acc);
         __syncthreads();
-        if (w == 0) q_pair_store_from(p, pk, job, l, acc);
+        if (w == 0) {
+            if (job < njobs_a) q_pair_store_from(pa, pk, job, l, acc);
+            else q_pair_store_from(pb, pk, job - njobs_a, l, acc);
+        }
     }
 }
 
@@ -310,11 +337,13 @@ hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream)
 
 int mlap_finish_wgs(const MlapParams &p) { return p.n_heads * 2 * ((p.T + MLAP_XTOK - 1) / MLAP_XTOK); }
 
-hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider)
 {
     const int nblk = p.h / MLAP_XBLOCK;
     int ngroups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
     const int nslabs = p.q_lora / 128 + 5;
+    if (rider != nullptr && !mlap_takes_rider(p)) return hipErrorInvalidValue;
+    const MlapRider rd = rider != nullptr ? *rider : MlapRider{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact) {
         // prefill sizes: the sums over the hidden axis on the matrix cores, up to four partial sums per token
         // as many ranges as give about two workgroups per compute unit (one is resident at a time, by its LDS)
@@ -331,7 +360,8 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
         hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p, nslabs, ngroups);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
-        hipLaunchKernelGGL(mlap_xlinear_kernel, dim3((unsigned)(nslabs * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, nslabs, ngroups);
+        const int xslabs = nslabs + (rider != nullptr ? 1 : 0);
+        hipLaunchKernelGGL(mlap_xlinear_kernel, dim3((unsigned)(xslabs * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, xslabs, ngroups, rd);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -352,7 +382,9 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
         hipLaunchKernelGGL(qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
         return hipGetLastError();
     }
-    const int qjobs = qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);
+    const int qjobs_a = qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);
+    const QProj qr = {p.q_norm, rd.w_qb, rd.qpart, p.T, p.q_lora, rd.q_slabs, p.q_norm_scale, nullptr};
+    const int qjobs = qjobs_a + qr.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);
     // as many workgroups as fit at once (by their LDS), every one with the same number of jobs where possible
     const int steps = p.q_lora / QPROJ_KSPLIT / 32;
     const int lds = steps == 12 ? qproj_lds_bytes<6>() : (steps == 8 ? qproj_lds_bytes<4>() : qproj_lds_bytes<2>());
@@ -362,9 +394,9 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream)
     const int rounds = (qjobs + slots - 1) / slots;
     const dim3 qgrid((unsigned)((qjobs + rounds - 1) / rounds));
     switch (steps) {
-    case 4: hipLaunchKernelGGL(qproj_kernel<2>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
-    case 8: hipLaunchKernelGGL(qproj_kernel<4>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
-    case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp, qjobs); break;
+    case 4: hipLaunchKernelGGL(qproj_kernel<2>, qgrid, dim3(128), 0, stream, qp, qjobs_a, qr, qjobs); break;
+    case 8: hipLaunchKernelGGL(qproj_kernel<4>, qgrid, dim3(128), 0, stream, qp, qjobs_a, qr, qjobs); break;
+    case 12: hipLaunchKernelGGL(qproj_kernel<6>, qgrid, dim3(128), 0, stream, qp, qjobs_a, qr, qjobs); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

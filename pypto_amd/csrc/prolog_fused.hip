@@ -1,10 +1,13 @@
 // MLA prolog + lightning-indexer prolog as one operator (mla_indexer_prolog_quant_d/_p of the reference,
-// examples/models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:141-256): the kernels of the two prologs in
-// the order hidden-axis sums -> norms and quantisation of the latents -> int8 projection of the attention query ->
-// first launch of the indexer prolog, and then ONE last launch for both: the workgroups that finish the attention
-// query (absorb product, 70 KB of LDS, four waves) and those that finish the indexer's query rows, key row and
-// weights (54 KB, eight waves) do not depend on each other and fit a compute unit together, so they run side by
-// side instead of one launch after the other.
+// examples/models/deepseek_v32_exp/mla_indexer_prolog_quant_impl.py:141-256).  At decode sizes it is the MLA
+// prolog's four launches with the indexer prolog's work riding in them (MlapRider): hidden-axis sums (wk as one
+// more column slab, w_proj beside the rope columns of w_dkv_kr) -> norms and quantisation of the latents -> int8
+// projections of the attention query and of the indexer query, jobs of one kind -> ONE last launch for both: the
+// workgroups that finish the attention query (absorb product, 70 KB of LDS, four waves) and those that finish the
+// indexer's query rows, key row and weights (54 KB, eight waves) do not depend on each other and fit a compute
+// unit together, so they run side by side instead of one launch after the other.  Where the indexer prolog cannot
+// ride (other than 64 indexer heads) its first launch follows the MLA prolog's third; at prefill sizes every stage
+// has a launch of its own.
 #include "prolog_finish.h"
 
 #include "prolog_fused.h"
@@ -33,6 +36,22 @@ __global__ __launch_bounds__(64 * FIN_WAVES) void prolog_fused_finish_kernel(con
 
 hipError_t prolog_fused_launch(const MlapParams &pm, const LipParams &pl, hipStream_t stream)
 {
+    // Decode sizes: the indexer prolog's first launch has no work of a kind of its own -- its sums over the hidden
+    // axis are more column slabs of the MLA prolog's first launch and its int8 projection more jobs of the third
+    // (MlapRider) -- so the pass is four launches: hidden-axis sums, latents, projections, one finish for both.
+    if (mlap_takes_rider(pm) && pl.T == pm.T && pl.h == pm.h && pl.q_lora == pm.q_lora && pl.x == pm.x && pl.q_norm == pm.q_norm &&
+        pl.q_norm_scale == pm.q_norm_scale && pl.n_heads == 64 && !lip_q_on_matrix_cores(pl)) {
+        const MlapRider rd = {pl.wk, pl.w_proj, pl.xpart, pl.w_qb, pl.qpart, pl.n_heads};
+        hipError_t e = mlap_launch_front(pm, stream, &rd);
+        if (e != hipSuccess) return e;
+        LipParams pg = pl;
+        pg.x_in_groups = 1;
+        const int mla_wgs = mlap_finish_wgs(pm);
+        const int q_wgs = lip_finish_query_wgs(pg);
+        hipLaunchKernelGGL(prolog_fused_finish_kernel, dim3((unsigned)(mla_wgs + q_wgs + pg.T)), dim3(64 * FIN_WAVES), 0, stream, pm, pg,
+                           mla_wgs, q_wgs);
+        return hipGetLastError();
+    }
     hipError_t e = mlap_launch_front(pm, stream);
     if (e != hipSuccess) return e;
     e = lip_launch_linear(pl, stream);

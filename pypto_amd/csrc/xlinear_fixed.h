@@ -30,6 +30,12 @@ struct XlSlab {
     int wbytes;           // bytes of a row that belong to the slab: 16, 32, 64, 128 or 256
     float *out;           // group sums of this group: out[t * out_pitch + column of the slab]
     int out_pitch;
+    // xl_body only: a 256-byte slab may be two 128-byte halves of different matrices.  With w_hi set (wbytes = 256),
+    // bytes 128..255 of a staged row are bytes 0..127 of w_hi's row, and columns 64..127 go to out_hi[t * out_pitch_hi + column - 64].
+    const uint8_t *w_hi = nullptr;
+    int pitch_hi = 0;
+    float *out_hi = nullptr;
+    int out_pitch_hi = 0;
 };
 
 // row widths the staging handles (whole 16-byte pieces, a power of two of them per row)
@@ -57,9 +63,11 @@ __device__ __forceinline__ void xl_body(const XlSlab &sl, const uint16_t *x, con
         {   // rows of wbytes bytes: wbytes/16 lanes per row
             const int lpr = wbytes >> 4;
             const int rpi = 64 / lpr;                                     // rows per request
-            const uint8_t *src = sl.w + (size_t)(k0 + l / lpr) * sl.pitch + 16 * (l % lpr);
+            const bool hi = sl.w_hi != nullptr && (l & 15) >= 8;          // this lane's piece belongs to the second matrix
+            const size_t pitch = hi ? sl.pitch_hi : sl.pitch;
+            const uint8_t *src = (hi ? sl.w_hi - 128 : sl.w) + (size_t)(k0 + l / lpr) * pitch + 16 * (l % lpr);
 #pragma unroll 1
-            for (int i = 0; i < XL_BLOCK / rpi; ++i) dma16(src + (size_t)i * rpi * sl.pitch, wdst + 1024 * i);
+            for (int i = 0; i < XL_BLOCK / rpi; ++i) dma16(src + (size_t)i * rpi * pitch, wdst + 1024 * i);
         }
 #pragma unroll
         for (int u = 0; u < XL_TOK / 2; ++u) {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + 2u + l/32
@@ -109,7 +117,9 @@ __device__ __forceinline__ void xl_body(const XlSlab &sl, const uint16_t *x, con
                 s1 = __fadd_rn(s1, v[1]);
             }
             f32x2 v = {s0, s1};
-            *reinterpret_cast<f32x2 *>(sl.out + (size_t)t * sl.out_pitch + 2 * l) = v;
+            float *dst = sl.out + (size_t)t * sl.out_pitch + 2 * l;
+            if (sl.w_hi != nullptr && l >= 32) dst = sl.out_hi + (size_t)t * sl.out_pitch_hi + 2 * l - 64;
+            *reinterpret_cast<f32x2 *>(dst) = v;
         }
     }
 }

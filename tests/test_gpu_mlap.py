@@ -193,11 +193,15 @@ def run_fused(dm, dl, t, n, n_idx, op=None):
     return q_nope, q_rope, q_int8, q_scale, weights
 
 
-@pytest.mark.parametrize("mode,shape", [("default", "small"), ("exact", "small"), ("matrix_cores", "small"), ("default", "t_512")])
+@pytest.mark.parametrize("mode,shape", [("default", "small"), ("exact", "small"), ("matrix_cores", "small"), ("default", "t_512"),
+                                        ("default", "t_11_idx_64"), ("exact", "t_11_idx_64"), ("default", "t_3_idx_32")])
 def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, shape):
     """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
     projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
-    indexer prolog called one after the other on the same inputs, bit for bit, in each of the summation modes."""
+    indexer prolog called one after the other on the same inputs, bit for bit, in each of the summation modes.
+    The two decode-sized shapes: with 64 indexer heads the indexer prolog's first stage rides in the MLA prolog's
+    launches (11 tokens: two token groups, the second ragged; 576 hidden channels: a second, short group of
+    blocks), with 32 heads it keeps its own launch."""
     from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd import mla_prolog_quant_impl as impl
     from pypto_amd.synthetic import gen_indexer_prolog_inputs
@@ -206,6 +210,12 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, sha
     if shape == "small":
         kw = dict(h=256, q_lora_rank=512)
         b, s1, act, n_mla, n_idx = 3, 50, [700, 650, 600], 4, 8
+    elif shape == "t_11_idx_64":
+        kw = dict(h=576, q_lora_rank=512)
+        b, s1, act, n_mla, n_idx = 11, 1, [700 - 37 * i for i in range(11)], 4, 64
+    elif shape == "t_3_idx_32":
+        kw = dict(h=576, q_lora_rank=512)
+        b, s1, act, n_mla, n_idx = 3, 1, [700, 650, 600], 4, 32
     else:   # the reference's test_t_512_tilebs_128_p (deepseekv32_mla_indexer_prolog_quant.py:1050-1117) at the model's sizes
         kw = {}
         b, s1, act, n_mla, n_idx = 128, 4, [4096] * 128, 128, 64
