@@ -20,8 +20,8 @@
 //                       quarter of the reduction axis, block of 32 tokens), one half each: the tile of
 //                       w_qb (rows x 128 bytes) and the token rows travel to LDS by LDS-DMA, all
 //                       requests issued up front; 32-row steps are consumed as their requests land
-//                       (they complete in order): 4x4 byte transposes (v_perm_b32) turn the row-major
-//                       tile into v_mfma_i32_32x32x32_i8 operands.  The two halves are added through
+//                       (they complete in order): the transposing 8-bit LDS read (ds_read_b64_tr_b8, two per
+//                       product) turns the row-major tile into v_mfma_i32_32x32x32_i8 operands.  The two halves are added through
 //                       LDS and the partial int32 sums go to the workspace.  The other two waves take
 //                       hidden-axis jobs (block of 64 rows of wk or of w_proj, 4 tokens): fp32 FMAs
 //                       with the hidden states as scalar operands; block sums go to the workspace.

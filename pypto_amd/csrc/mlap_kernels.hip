@@ -21,7 +21,7 @@
 //                        int8 quantisation of the query latent; RMS norm and per-slab quantisation of
 //                        the key latent, rope of the key, scatter into the caches.
 //   qproj_kernel         int8 projection of the query latent (shared job code: LDS-DMA tile,
-//                        v_perm_b32 transposes, v_mfma_i32_32x32x32_i8), partial sums per quarter.
+//                        transposing 8-bit LDS reads, v_mfma_i32_32x32x32_i8), partial sums per quarter.
 //   mlap_finish_kernel   per (head, half of the 512 output columns, 8 tokens): partial sums added and
 //                        de-quantised, rope part rotated and stored, nope part times the head's w_uk
 //                        slice (staged in LDS by LDS-DMA): on the matrix cores, or one output column per lane.
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj pa, const int nj
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][r] = 0;
         const uint8_t *region = bufs + (k & 1) * BUF;
-#pragma unroll 1
+#pragma unroll
         for (int s = 0; s < HS; ++s) q_step<HS>(region, s, l, acc);
         uint8_t *pk = park + (k & 1) * LIN_RED_BYTES;
         if (w == 1) q_pair_park(pk, l, acc);

@@ -45,32 +45,45 @@ __device__ __forceinline__ void wait_vm_le(const int n)
     }
 }
 
-// rows d0..d3 of four bytes each -> columns o0..o3 (o_i = byte i of d0, d1, d2, d3)
-__device__ __forceinline__ void transpose4x4(const uint32_t d0, const uint32_t d1, const uint32_t d2, const uint32_t d3,
-                                             uint32_t &o0, uint32_t &o1, uint32_t &o2, uint32_t &o3)
-{
-    const uint32_t t0 = __builtin_amdgcn_perm(d1, d0, 0x05010400u);
-    const uint32_t t1 = __builtin_amdgcn_perm(d1, d0, 0x07030602u);
-    const uint32_t u0 = __builtin_amdgcn_perm(d3, d2, 0x05010400u);
-    const uint32_t u1 = __builtin_amdgcn_perm(d3, d2, 0x07030602u);
-    o0 = __builtin_amdgcn_perm(u0, t0, 0x05040100u);
-    o1 = __builtin_amdgcn_perm(u0, t0, 0x07060302u);
-    o2 = __builtin_amdgcn_perm(u1, t1, 0x05040100u);
-    o3 = __builtin_amdgcn_perm(u1, t1, 0x07060302u);
-}
-
 __device__ __forceinline__ float bf16_round_f32(const float v)
 {
     return __uint_as_float(pack_bf16x2(v, 0.0f) << 16);
+}
+
+// Weight operands by the transposing 8-bit LDS read.  ds_read_b64_tr_b8 takes, per group of
+// 16 lanes, the 16 rows of 8 bytes its lanes point at and hands lane j byte j of the even lanes' rows and lane 8 + j
+// byte j of the odd lanes' rows.  Even lanes point at eight consecutive rows of the tile at one block of 8 columns,
+// odd lanes at the same rows of the next block: lane n of the group then holds column n of 16, eight rows deep --
+// half of what v_mfma_i32_32x32x32_i8 wants from a lane (column l % 32, rows 16*(l / 32) .. +15), so two reads per
+// product and no byte shuffling.  Product i covers columns 32*i .. 32*i + 31 of the slab.
+// Tile layout the reads assume: row r (128 bytes) keeps its 16-byte piece q at piece q ^ 2*((r >> 1) & 3), so that
+// the eight rows of a half-wave's read fall on different banks; the LDS-DMA requests place the pieces that way.
+__device__ __forceinline__ int q_tr_piece_swizzle(const int row) { return 2 * ((row >> 1) & 3); }
+
+__device__ __forceinline__ void q_build_a_tr(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
+{
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    const int x = (l >> 2) & 3;                         // (row >> 1) & 3 of this lane's rows
+    const uint8_t *base = tile + (32 * s + 16 * (l >> 5) + ((l & 15) >> 1)) * 128 + 16 * ((l >> 4) & 1) + 8 * (l & 1);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint8_t *pi = base + 32 * (i ^ x);
+        const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)pi);
+        const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)(pi + 8 * 128));
+        a[i][0] = lo[0];
+        a[i][1] = lo[1];
+        a[i][2] = hi[0];
+        a[i][3] = hi[1];
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
 // Int8 projection [T, q_lora] x [q_lora, 128*nslabs] -> partial int32 sums: one job per (slab of 128 columns, quarter of the reduction axis, block of 32 tokens); its
 // waves 0 and 1 take one half of the quarter each (HS steps of 32 rows).
 // LDS region of a wave: [tile: 32*HS rows x 128 bytes][token operands: HS x 1024 bytes].
-// Matrix product per step: A = 32 output columns x 32 rows of the tile (lane (j, g) holds rows
-// 16g..16g+15 of column 4j+i for product i), B = 32 tokens x the same 32 rows of q_norm, so that
-// accumulator register r of lane l holds column 4*(8*(r/4) + 4*(l/32) + r%4) + i, token l%32.
+// Matrix product per step: A = 32 output columns x 32 rows of the tile (product i: columns 32i .. 32i+31; lane l
+// holds rows 16*(l/32) .. +15 of column 32i + l%32, q_build_a_tr), B = 32 tokens x the same 32 rows of q_norm, so
+// that accumulator registers 4*rg .. 4*rg+3 of product i hold columns 32i + 8*rg + 4*(l/32) .. +3 of token l%32.
 template <int HS>
 __device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const int job, const int half)
 {
@@ -94,47 +107,23 @@ __device__ __forceinline__ void q_issue(const QProj &p, uint8_t *region, const i
 #pragma unroll 1
         for (int s = 0; s < HS; ++s) dma16(src + 32 * s, tok + 1024 * s);
     }
-    {   // rows 16..31 of every step are staged with neighbours swapped (q_step_at)
-        const int8_t *src = p.w + ((size_t)k0 + (l >> 3)) * ncols + head * 128 + 16 * (l & 7);
-        const int8_t *swp = p.w + ((size_t)k0 + ((l >> 3) ^ 1)) * ncols + head * 128 + 16 * (l & 7);
+    {   // lane l fills piece l % 8 of row l / 8 of a request's eight rows, with the piece q_build_a_tr expects there
+        const int8_t *src = p.w + ((size_t)k0 + (l >> 3)) * ncols + head * 128 + 16 * ((l & 7) ^ q_tr_piece_swizzle(l >> 3));
 #pragma unroll 1
         for (int i = 0; i < NW; i += 4) {
             dma16(src + (size_t)i * 8 * ncols, tile + 1024 * i);
             dma16(src + (size_t)(i + 1) * 8 * ncols, tile + 1024 * (i + 1));
-            dma16(swp + (size_t)(i + 2) * 8 * ncols, tile + 1024 * (i + 2));
-            dma16(swp + (size_t)(i + 3) * 8 * ncols, tile + 1024 * (i + 3));
+            dma16(src + (size_t)(i + 2) * 8 * ncols, tile + 1024 * (i + 2));
+            dma16(src + (size_t)(i + 3) * 8 * ncols, tile + 1024 * (i + 3));
         }
     }
 }
 
-// one 32-row step of the product: rows 32s.. of the tile, token operands of step s at tok + 1024 s.  Lanes 0..31
-// read rows 0..15 of the step, lanes 32..63 rows 16..31; a row is 32 dwords, so rows of the same parity share their
-// banks: rows 16..31 sit in LDS with neighbours swapped (row 16 + r at 16 + (r ^ 1)), which puts the two half-waves
-// of a read on opposite halves of the banks.
-// the four weight operands of step s (32 output columns each) from the tile
-__device__ __forceinline__ void q_build_a(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
-{
-    const uint32_t *tile32 = reinterpret_cast<const uint32_t *>(tile);
-    const int hi = l >> 5;
-    const int rd = (16 * hi) * 32 + (l & 31);           // dword index of this lane's first row of a step
-    const int rd_even = rd + 32 * hi, rd_odd = rd - 32 * hi;
-    uint32_t d[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) d[r] = tile32[s * 32 * 32 + ((r & 1) ? rd_odd : rd_even) + r * 32];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        uint32_t o0, o1, o2, o3;
-        transpose4x4(d[4 * q], d[4 * q + 1], d[4 * q + 2], d[4 * q + 3], o0, o1, o2, o3);
-        a[0][q] = (int)o0;
-        a[1][q] = (int)o1;
-        a[2][q] = (int)o2;
-        a[3][q] = (int)o3;
-    }
-}
+// one 32-row step of the product: rows 32s.. of the tile, token operands of step s at tok + 1024 s
 __device__ __forceinline__ void q_step_at(const uint8_t *tile, const uint8_t *tok, const int s, const int l, i32x16 (&acc)[4])
 {
     i32x4 a[4];
-    q_build_a(tile, s, l, a);
+    q_build_a_tr(tile, s, l, a);
     const i32x4 b = *reinterpret_cast<const i32x4 *>(tok + 1024 * s + 16 * l);
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
@@ -181,12 +170,13 @@ __device__ __forceinline__ void q_pair_store_from(const QProj &p, const uint8_t 
     if (t < p.T) {
         int32_t *dst = p.part + ((size_t)kq * p.T + t) * ncols + head * 128;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = 8 * (r >> 2) + 4 * (l >> 5) + (r & 3);
-            const i32x4 o = red[r * 64 + l];
-            i32x4 v = {acc[0][r] + o[0], acc[1][r] + o[1], acc[2][r] + o[2], acc[3][r] + o[3]};
-            *reinterpret_cast<i32x4 *>(dst + 4 * m) = v;
-        }
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const i32x4 o = red[(4 * i + rg) * 64 + l];
+                i32x4 v = {acc[i][4 * rg] + o[0], acc[i][4 * rg + 1] + o[1], acc[i][4 * rg + 2] + o[2], acc[i][4 * rg + 3] + o[3]};
+                *reinterpret_cast<i32x4 *>(dst + 32 * i + 8 * rg + 4 * (l >> 5)) = v;
+            }
     }
 }
 // the same with wave 1's accumulators parked in its own (consumed) tile region, the second of two
@@ -200,37 +190,12 @@ __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const 
 {
     i32x4 *red = reinterpret_cast<i32x4 *>(region);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        i32x4 v = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-        red[r * 64 + l] = v;
-    }
-}
-
-// Weight operands for the unsplit forms by the transposing 8-bit LDS read.  ds_read_b64_tr_b8 takes, per group of
-// 16 lanes, the 16 rows of 8 bytes its lanes point at and hands lane j byte j of the even lanes' rows and lane 8 + j
-// byte j of the odd lanes' rows.  Even lanes point at eight consecutive rows of the tile at one block of 8 columns,
-// odd lanes at the same rows of the next block: lane n of the group then holds column n of 16, eight rows deep --
-// half of what v_mfma_i32_32x32x32_i8 wants from a lane (column l % 32, rows 16*(l / 32) .. +15), so two reads per
-// product and no byte shuffling.  Product i covers columns 32*i .. 32*i + 31 of the slab.
-// Tile layout the reads assume: row r (128 bytes) keeps its 16-byte piece q at piece q ^ 2*((r >> 1) & 3), so that
-// the eight rows of a half-wave's read fall on different banks; the LDS-DMA requests place the pieces that way.
-__device__ __forceinline__ int q_tr_piece_swizzle(const int row) { return 2 * ((row >> 1) & 3); }
-
-__device__ __forceinline__ void q_build_a_tr(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
-{
-    typedef int v2i __attribute__((ext_vector_type(2)));
-    const int x = (l >> 2) & 3;                         // (row >> 1) & 3 of this lane's rows
-    const uint8_t *base = tile + (32 * s + 16 * (l >> 5) + ((l & 15) >> 1)) * 128 + 16 * ((l >> 4) & 1) + 8 * (l & 1);
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint8_t *pi = base + 32 * (i ^ x);
-        const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)pi);
-        const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)(pi + 8 * 128));
-        a[i][0] = lo[0];
-        a[i][1] = lo[1];
-        a[i][2] = hi[0];
-        a[i][3] = hi[1];
-    }
+        for (int rg = 0; rg < 4; ++rg) {
+            i32x4 v = {acc[i][4 * rg], acc[i][4 * rg + 1], acc[i][4 * rg + 2], acc[i][4 * rg + 3]};
+            red[(4 * i + rg) * 64 + l] = v;
+        }
 }
 
 // The unsplit forms' results leave de-quantised, as bf16, through a staging area of the wave's own in LDS
