@@ -15,7 +15,11 @@ constexpr int MLAP_MAX_XGROUPS = 32; // h <= 32 * 8 * 64 = 16384
 constexpr int MLAP_MAX_QLORA = 1536;
 constexpr int QPROJ_KSPLIT_HOST = 4; // partial sums of the int8 projection (prolog_common.h: QPROJ_KSPLIT)
 constexpr int MLAP_XTOK = 8;         // tokens per job of the first and of the last kernel
-constexpr int MLAP_MFMA_MIN_TOKENS = 64;   // from here on the first launch sums on the matrix cores (unless absorb_exact)
+constexpr int MLAP_MFMA_MIN_TOKENS = 16;   // from here on the stages take their prefill forms unless absorb_exact: the first launch
+                                           // sums on the matrix cores, the projection runs unsplit, the last stage walks token blocks
+                                           // per head (at 16 tokens the decode forms, whose cost grows with every 8 tokens, have
+                                           // caught up with the flat cost of those forms)
+constexpr int MLAP_UNSPLIT_MIN_TOKENS = 64;   // with absorb_exact the projection still runs unsplit from here on
 constexpr int MLAP_XM_MAX_SPLITS = 8;      // ranges of the hidden axis (partial sums per token) of that form, at most
 
 // rows [T, q_lora + 576] of partial sums over the hidden axis the workspace holds: the group sums of the
@@ -71,8 +75,15 @@ struct MlapRider {
     int q_slabs;
 };
 
-// whether the launches of `p` take a rider at all: the decode form only
-inline bool mlap_takes_rider(const MlapParams &p) { return p.T < MLAP_MFMA_MIN_TOKENS; }
+// the stages' prefill forms (matrix-core sums over the hidden axis, last stage per head and run of token blocks)
+__host__ __device__ inline bool mlap_prefill_forms(const MlapParams &p) { return p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact; }
+// partial sums per output the int8 projection leaves: 1 = unsplit (de-quantised bf16), else QPROJ_KSPLIT_HOST int32 partials
+__host__ __device__ inline int mlap_qsplits(const MlapParams &p)
+{
+    return (mlap_prefill_forms(p) || p.T >= MLAP_UNSPLIT_MIN_TOKENS) ? 1 : QPROJ_KSPLIT_HOST;
+}
+// whether the launches of `p` take a rider at all: the decode forms only
+inline bool mlap_takes_rider(const MlapParams &p) { return !mlap_prefill_forms(p) && mlap_qsplits(p) != 1; }
 
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
 // all launches but the last, and the number of workgroups of the last (for the fused operator's last launch)

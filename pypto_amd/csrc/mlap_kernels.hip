@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapP
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill form of the first launch: the same product on the matrix cores (xlinear_mfma.h), for 64 tokens and more
+// Prefill form of the first launch: the same product on the matrix cores (xlinear_mfma.h), for MLAP_MFMA_MIN_TOKENS tokens and more
 // when the caller has not asked for the fixed-order sums.  workgroup = (slab of 128 columns of [w_dq | w_dkv_kr],
 // one of nsplit ranges of the hidden axis, 128 tokens); the 64 rope columns are a narrow slab of their own.
 static_assert(XM_KC == MLAP_XBLOCK, "the workspace is sized in chunks of the hidden axis");
@@ -318,7 +318,7 @@ __global__ __launch_bounds__(64 * FINP_WAVES) void mlap_finish_prefill_kernel(co
 
 }  // namespace
 
-bool mlap_finish_is_prefill(const MlapParams &p) { return p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact; }
+bool mlap_finish_is_prefill(const MlapParams &p) { return mlap_prefill_forms(p); }
 
 hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream)
 {
@@ -344,7 +344,7 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
     const int nslabs = p.q_lora / 128 + 5;
     if (rider != nullptr && !mlap_takes_rider(p)) return hipErrorInvalidValue;
     const MlapRider rd = rider != nullptr ? *rider : MlapRider{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
-    if (p.T >= MLAP_MFMA_MIN_TOKENS && !p.absorb_exact) {
+    if (mlap_prefill_forms(p)) {
         // prefill sizes: the sums over the hidden axis on the matrix cores, up to four partial sums per token
         // as many ranges as give about two workgroups per compute unit (one is resident at a time, by its LDS)
         const int nchunks = p.h / XM_KC;
@@ -369,7 +369,7 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128, p.q_norm_scale, p.w_qb_scale};
-    if (qproj_splits(p.T) == 1) {
+    if (mlap_qsplits(p) == 1) {
         if (p.q_lora % (32 * QPF_STEPS)) return hipErrorInvalidValue;
         const int cus = cu_count();
         if (cus <= 0) return hipErrorNoDevice;

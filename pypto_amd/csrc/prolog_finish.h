@@ -14,10 +14,10 @@ namespace {
 
 // the de-quantised int8 projection for columns col, col + 1 of token t, as bf16-valued floats: the unsplit form left
 // them that way; the split form's partial sums are added and de-quantised here
-__device__ __forceinline__ void q_value2(const int32_t *part, const int T, const int t, const int ncols, const int col, const float ts,
-                                         const float cs0, const float cs1, float &v0, float &v1)
+__device__ __forceinline__ void q_value2(const int32_t *part, const int splits, const int T, const int t, const int ncols, const int col,
+                                         const float ts, const float cs0, const float cs1, float &v0, float &v1)
 {
-    if (qproj_splits(T) == 1) {
+    if (splits == 1) {
         const uint32_t v = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(part) + (size_t)t * ncols + col);
         v0 = __uint_as_float(v << 16);
         v1 = __uint_as_float(v & 0xffff0000u);
@@ -178,7 +178,7 @@ __device__ __forceinline__ void lip_finish_body(const LipParams &p, const int q_
         const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
         const uint32_t rc = rope_coef(p.cos, t, l), rs = rope_coef(p.sin, t, l);
         float v0, v1;
-        q_value2(p.qpart, p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
+        q_value2(p.qpart, qproj_splits(p.T), p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
         rope_pair(v0, v1, rc, rs, l);
         f32x2 av = {v0, v1};
         *reinterpret_cast<f32x2 *>(&arow[w][2 * l]) = av;
@@ -499,7 +499,7 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
             const int col = head * MLAP_QHEAD + 2 * l;
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
             float av0, av1;
-            q_value2(p.qpart, p.T, tt, ncols, col, ts, cs[0], cs[1], av0, av1);
+            q_value2(p.qpart, mlap_qsplits(p), p.T, tt, ncols, col, ts, cs[0], cs[1], av0, av1);
             const f32x2 av = {av0, av1};
             *reinterpret_cast<f32x2 *>(&arow[tl][2 * l]) = av;
             *reinterpret_cast<uint32_t *>(&abf[tl][2 * l]) = pack_bf16x2(av[0], av[1]);
@@ -509,7 +509,7 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
             const int col = head * MLAP_QHEAD + MLAP_NOPE + 2 * l;
             const f32x2 cs = *reinterpret_cast<const f32x2 *>(p.w_qb_scale + col);
             float v0, v1;
-            q_value2(p.qpart, p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
+            q_value2(p.qpart, mlap_qsplits(p), p.T, t, ncols, col, ts, cs[0], cs[1], v0, v1);
             const float c0 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + l]), c1 = bf16_bits_to_f32(p.cos[(size_t)t * MLAP_ROPE + 32 + l]);
             const float sn0 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + l]), sn1 = bf16_bits_to_f32(p.sin[(size_t)t * MLAP_ROPE + 32 + l]);
             const float r0 = __builtin_fmaf(v0, c0, (-v1) * sn0);
@@ -603,7 +603,7 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
 }
 
 // ------------------------------------------------------------------------ MLA prolog, prefill sizes
-// The same last stage for 64 tokens and more with the absorb product on the matrix cores: one workgroup of eight
+// The same last stage for MLAP_MFMA_MIN_TOKENS tokens and more with the absorb product on the matrix cores: one workgroup of eight
 // waves per (head, run of `per` blocks of 32 tokens).  The head's whole w_uk (128 x 512 bf16, 128 KiB) is staged
 // once, wave w keeping the slice of output columns 64w..64w+63 in the layout of the decode form; then per block:
 // wave w moves the query channels of tokens 4w..4w+3 (de-quantised bf16 already: the projection is unsplit at these
@@ -616,7 +616,6 @@ constexpr int FINP_APITCH = MLAP_NOPE + 8;   // elements between operand rows: 2
 constexpr int FINP_SPITCH = 144;             // bytes between the rows of a wave's output staging area (8 tokens x 64 columns)
 constexpr int FINP_STAGE = 8 * FINP_SPITCH;
 constexpr int MLAP_FINP_LDS = FINP_WAVES * FIN_W_BYTES + 2 * FINP_TOK * FINP_APITCH * 2 + FINP_WAVES * FINP_STAGE;   // 157 696 bytes
-static_assert(MLAP_MFMA_MIN_TOKENS >= QPROJ_PREFILL_TOKENS, "the prefill form reads one partial sum per output");
 
 struct FinRaw {
     uint32_t nope[4], rope[4];     // two bf16 values each: the unsplit projection leaves its results de-quantised
