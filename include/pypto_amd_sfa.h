@@ -386,8 +386,8 @@ typedef struct PtoMlaPrologQuantArgs {
                              above); 0 = on the matrix cores: the same exact bf16 products summed in fp32 in the
                              cores' order, so some results differ in the last bf16 bit -- inside the reference's
                              own acceptance rule for this output (deepseekv32_mla_prolog_quant.py:668-692), which
-                             only feeds the attention.  With fewer than 16 tokens every other output is the same either
-                             way; from 16 tokens on, 0 also takes the sums over the hidden axis on the matrix cores
+                             only feeds the attention.  With at most 8 tokens every other output is the same either
+                             way; from 9 tokens on, 0 also takes the sums over the hidden axis on the matrix cores
                              (int8 latents then differ by one step in rare entries, inside the same rule) and 1
                              keeps every sum in its fixed order. */
     int32_t reserved;

@@ -15,10 +15,10 @@ constexpr int MLAP_MAX_XGROUPS = 32; // h <= 32 * 8 * 64 = 16384
 constexpr int MLAP_MAX_QLORA = 1536;
 constexpr int QPROJ_KSPLIT_HOST = 4; // partial sums of the int8 projection (prolog_common.h: QPROJ_KSPLIT)
 constexpr int MLAP_XTOK = 8;         // tokens per job of the first and of the last kernel
-constexpr int MLAP_MFMA_MIN_TOKENS = 16;   // from here on the stages take their prefill forms unless absorb_exact: the first launch
+constexpr int MLAP_MFMA_MIN_TOKENS = 9;    // from here on the stages take their prefill forms unless absorb_exact: the first launch
                                            // sums on the matrix cores, the projection runs unsplit, the last stage walks token blocks
-                                           // per head (at 16 tokens the decode forms, whose cost grows with every 8 tokens, have
-                                           // caught up with the flat cost of those forms)
+                                           // per head (the decode forms work on 8 tokens at a time and their cost grows with every
+                                           // 8 tokens; those forms cost the same from 9 to 128 tokens, about what 8 tokens cost here)
 constexpr int MLAP_UNSPLIT_MIN_TOKENS = 64;   // with absorb_exact the projection still runs unsplit from here on
 constexpr int MLAP_XM_MAX_SPLITS = 8;      // ranges of the hidden axis (partial sums per token) of that form, at most
 

@@ -19,7 +19,7 @@ is copied first).  Returns ``None``; runs asynchronously on the current stream.
 matrix cores (the default: the same exact bf16 products, fp32 sums in the cores' order, so some results differ in
 the last bf16 bit from the sequential statement -- inside the reference's own acceptance rule for this output,
 deepseekv32_mla_prolog_quant.py:668-692) or, when ``True``, as fixed-order fp32 sums that reproduce the
-sequential statement bit for bit.  Every other output is the same either way for fewer than 16 tokens; from 16 tokens
+sequential statement bit for bit.  Every other output is the same either way for at most 8 tokens; from 9 tokens
 on (larger decode batches, prefill chunks) the default also takes the sums over the hidden axis (``x . w_dq``, ``x . w_dkv_kr``) on the matrix
 cores -- sixteen times faster at 512 tokens, the int8 latents then differ by one step in rare entries, inside
 the same acceptance rule -- and ``EXACT_ABSORB = True`` keeps every sum in its fixed order.

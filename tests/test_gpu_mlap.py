@@ -98,7 +98,7 @@ def test_mla_prolog_matrix_core_absorb_default():
     differs from it by at most one bf16 step."""
     from pypto_amd import mla_prolog_quant_impl as impl
     impl.EXACT_ABSORB = False
-    for b, s1, act, kw in ((4, 2, [4096] * 4, {}), (5, 3, [900] * 5, dict(h=192, q_lora_rank=512, n_heads=2))):   # 8 and 15 tokens
+    for b, s1, act, kw in ((4, 2, [4096] * 4, {}), (2, 3, [900] * 2, dict(h=192, q_lora_rank=512, n_heads=2))):   # 8 and 6 tokens
         inp = gen_mla_prolog_inputs(b, s1, act, seed=31 + b, **kw)
         ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
         got = run_op(inp, (1e-5, 1e-5))
@@ -121,17 +121,17 @@ def test_mla_prolog_prefill_t512():
 
 
 def test_mla_prolog_prefill_t512_matrix_core_sums_default():
-    """The operator's default from 16 tokens on: the sums over the hidden axis run on the matrix cores as well
+    """The operator's default from 9 tokens on: the sums over the hidden axis run on the matrix cores as well
     (same exact products, the cores' own summation order), so the int8 latents may differ by one step where the
     sequential sums land next to a rounding boundary.  Held to the reference's acceptance rule for every output
     (deepseekv32_mla_prolog_quant.py:668-692) against the sequential statement; a short-h shape with ragged
     token tiles and a half-empty chunk split rides along, and the decode batches that take these forms: 16 and 32
-    tokens at the model's sizes, 39 and 63 (ragged blocks of 32) at small ones."""
+    tokens at the model's sizes, 9, 39 and 63 (ragged blocks of 32) at small ones."""
     from pypto_amd import mla_prolog_quant_impl as impl
     impl.EXACT_ABSORB = False
     small = dict(h=192, q_lora_rank=512, n_heads=2)
     for b, s1, act, kw in ((1, 512, [4096], {}), (3, 50, [700] * 3, small), (16, 1, [4096] * 16, {}), (32, 1, [4096] * 32, {}),
-                           (3, 13, [700] * 3, small), (9, 7, [300] * 9, small)):
+                           (3, 13, [700] * 3, small), (9, 7, [300] * 9, small), (9, 1, [300] * 9, small)):
         inp = gen_mla_prolog_inputs(b, s1, act, seed=41 + b, **kw)
         ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
         got = run_op(inp, (1e-5, 1e-5), prefill=True)
@@ -198,14 +198,14 @@ def run_fused(dm, dl, t, n, n_idx, op=None):
 
 @pytest.mark.parametrize("mode,shape", [("default", "small"), ("exact", "small"), ("matrix_cores", "small"), ("default", "t_512"),
                                         ("default", "t_11_idx_64"), ("exact", "t_11_idx_64"), ("default", "t_3_idx_32"),
-                                        ("default", "t_40_idx_64"), ("exact", "t_40_idx_64")])
+                                        ("default", "t_40_idx_64"), ("exact", "t_40_idx_64"), ("default", "t_7_idx_64")])
 def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, shape):
     """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
     projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
     indexer prolog called one after the other on the same inputs, bit for bit, in each of the summation modes.
     The two decode-sized shapes: with 64 indexer heads the indexer prolog's first stage rides in the MLA prolog's
-    launches (11 tokens: two token groups, the second ragged; 576 hidden channels: a second, short group of
-    blocks), with 32 heads it keeps its own launch.  At 40 tokens the MLA half takes its prefill forms by default
+    launches (7 tokens by default; 11 in the exact mode: two token groups, the second ragged; 576 hidden channels: a
+    second, short group of blocks), with 32 heads it keeps its own launch.  At 40 tokens the MLA half takes its prefill forms by default
     while the indexer half keeps its decode forms (in the exact mode both keep them, and the rider)."""
     from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd import mla_prolog_quant_impl as impl
@@ -218,6 +218,9 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, sha
     elif shape == "t_11_idx_64":
         kw = dict(h=576, q_lora_rank=512)
         b, s1, act, n_mla, n_idx = 11, 1, [700 - 37 * i for i in range(11)], 4, 64
+    elif shape == "t_7_idx_64":
+        kw = dict(h=576, q_lora_rank=512)
+        b, s1, act, n_mla, n_idx = 7, 1, [700 - 37 * i for i in range(7)], 4, 64
     elif shape == "t_40_idx_64":
         kw = dict(h=576, q_lora_rank=512)
         b, s1, act, n_mla, n_idx = 5, 8, [700, 650, 600, 550, 500], 4, 64
