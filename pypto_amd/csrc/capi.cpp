@@ -123,13 +123,29 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
     const int min_split = (int)((a->topk + pto::SFA_MAX_CHUNK - 1) / pto::SFA_MAX_CHUNK);
     int ns = a->num_splits;
     if (ns == 0) {
-        // fill the chip once; a split shorter than four tiles is all prologue
+        // The split count with the shortest schedule.  The workgroups of a row share an XCD (row t on XCD t % 8,
+        // for the row's queries in that XCD's L2) and a compute unit holds one workgroup, so the fullest XCD runs
+        // ceil(its workgroups / its CUs) rounds, each as long as a split's tiles plus the fixed cost of a workgroup
+        // (query staging, row table, first tile, writing the partial results: about five and a half tiles' time;
+        // three when nothing is split); the merge launch costs about a tile plus a tile per hundred partial rows.
+        // Filling every XCD exactly once wins where the batch allows it; a batch that does not divide the CUs
+        // gets fewer, longer splits rather than a second round that is nearly empty.  A split shorter than four
+        // tiles is all prologue.
         // (a size query on a host without a device plans for the 256 CUs of an MI355X; a launch there fails)
-        const long long wgs = rows * pl.hgroups;
         const int cus = cu_count() > 0 ? cu_count() : 256;
-        ns = (int)((cus + wgs - 1) / wgs);
+        const long long xcd_cus = cus / 8 > 0 ? cus / 8 : 1;
+        const long long xcd_rows = (rows + 7) / 8;
         const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
-        ns = ns > max_split ? max_split : ns;
+        double best = -1.0;
+        for (int s = 1; s <= max_split; ++s) {
+            const long long rounds = (xcd_rows * pl.hgroups * s + xcd_cus - 1) / xcd_cus;
+            const double merge = s == 1 ? 0.0 : 1.0 + 0.01 * (double)rows * s * pl.hgroups;
+            const double cost = (double)rounds * ((tiles + s - 1) / s + (s == 1 ? 3.0 : 5.5)) + merge;
+            if (best < 0.0 || cost < best) {
+                best = cost;
+                ns = s;
+            }
+        }
     }
     ns = ns < min_split ? min_split : ns;
     ns = ns > tiles ? tiles : ns;

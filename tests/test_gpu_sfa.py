@@ -105,6 +105,20 @@ def test_key_splits_agree_with_single_workgroup(splits):
     assert max_abs <= 2 ** -6
 
 
+@pytest.mark.parametrize("b", [20, 44])
+def test_batches_that_do_not_divide_the_compute_units(b):
+    """Batches whose rows do not spread evenly over the eight XCDs (20 rows: three on some, two on others; 44: six and
+    five): the library's own split count (fewer, longer splits instead of a second, nearly empty round of
+    workgroups) against the same launch with one workgroup per row, at the top-k of the benchmark."""
+    inp = gen_sfa_inputs(b, 1, 128, [4096 - 61 * i for i in range(b)], topk=2048, seed=b)
+    base = run_op(inp, num_splits=1)
+    out = run_op(inp)
+    max_abs, mean_rel = attention_error_stats(out, base)
+    print(f"b={b}: default splits vs one workgroup per row: max_abs={max_abs:.4g} mean_rel={mean_rel:.4g}", flush=True)
+    assert max_abs <= 2 ** -6
+    check(out, oracle(inp), f"b={b}, default splits")
+
+
 def test_prefill_entry_point_and_causal_rows():
     """Chunked-prefill shape in miniature: every query row t sees min(t+1, topk) keys."""
     inp = gen_sfa_inputs(1, 96, 128, [96], topk=64, seed=5)
