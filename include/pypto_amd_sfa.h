@@ -90,8 +90,9 @@ extern "C" {
  * Constraints: n_kv == 1, topk >= 1, block_size >= 1, nq >= 1.
  * Alignment: query, cache, output and workspace pointers 16 bytes (a contiguous
  * torch view with a storage offset may not be), the int32 tensors 4 bytes.
- * num_splits: how many workgroups share one query row's keys (0 = choose from
- * the device's compute-unit count).  When a row is split, each split's result
+ * num_splits: how many workgroups share one query row's keys (0 = the count
+ * that fills the device's compute units in one round of workgroups, or the
+ * nearest count below that when the batch does not divide them).  When a row is split, each split's result
  * travels as fp16 normalised by the split's own row sum: de-quantised cache
  * values must stay below 65504 in magnitude (always true of int8 * scale for
  * sane scales; for the bf16 cache of pto_sfa_bf16kv_launch larger values give
