@@ -307,8 +307,9 @@ def other_shapes_leg(torch, pypto_amd, dev):
 
 def prefill_prologs_leg(torch, pypto_amd, dev):
     """The two prologs at the reference's prefill-sized cases (MLA prolog b=1 s=512; indexer prolog b=128 s=4 and
-    b=1 s=4096): time per eager call, in the default summation mode and with the indexer's sums over the hidden
-    axis on the matrix cores."""
+    b=1 s=4096) and the MLA prolog at a decode batch of 32: time per eager call, in the default summation mode,
+    with every sum of the MLA prolog in its fixed order, and with the indexer's sums over the hidden axis on the
+    matrix cores."""
     from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
 
@@ -326,15 +327,23 @@ def prefill_prologs_leg(torch, pypto_amd, dev):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n * 1e3
     res = []
-    d = gen_mla_prolog_inputs(1, 512, [4096], seed=0).to(dev)
-    t, n, ql = 512, 128, 1536
-    outs = (torch.empty([t, ql], dtype=torch.int8, device=dev), torch.empty([t, 1], dtype=torch.float32, device=dev),
-            torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev), torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev),
-            d.kv_cache, d.kr_cache, d.k_scale_cache)
-    ins = list(d.input_tensors())
-    res.append({"operator": "mla_prolog_quant_p", "tokens": t, "sums": "default",
-                "us_per_call": timed(lambda: pypto_amd.mla_prolog_quant_p(*ins, *outs, 1e-5, 1e-5, "PA_BSND", None, None))})
-    del d, outs, ins
+    from pypto_amd import mla_prolog_quant_impl as mla_impl
+    # the MLA prolog at the batch of configs[2] (32 sequences, one token each) in both summation modes -- the default
+    # takes the prefill forms from 9 tokens on, the exact mode keeps the decode forms up to 63 -- and at 512 tokens
+    for b, s1, exact in ((32, 1, False), (32, 1, True), (1, 512, False)):
+        d = gen_mla_prolog_inputs(b, s1, [4096] * b, seed=0).to(dev)
+        t, n, ql = b * s1, 128, 1536
+        outs = (torch.empty([t, ql], dtype=torch.int8, device=dev), torch.empty([t, 1], dtype=torch.float32, device=dev),
+                torch.empty([t, n, 512], dtype=torch.bfloat16, device=dev), torch.empty([t, n, 64], dtype=torch.bfloat16, device=dev),
+                d.kv_cache, d.kr_cache, d.k_scale_cache)
+        ins = list(d.input_tensors())
+        mla_impl.EXACT_ABSORB = exact
+        try:
+            us = timed(lambda: pypto_amd.mla_prolog_quant_p(*ins, *outs, 1e-5, 1e-5, "PA_BSND", None, None))
+        finally:
+            mla_impl.EXACT_ABSORB = False
+        res.append({"operator": "mla_prolog_quant_p", "tokens": t, "sums": "every sum in its fixed order" if exact else "default", "us_per_call": us})
+        del d, outs, ins
     for b, s1, act in ((128, 4, [8192] * 128), (1, 4096, [65536])):
         d = gen_indexer_prolog_inputs(b, s1, act, seed=0).to(dev)
         t, n = b * s1, d.w_proj.shape[1]
