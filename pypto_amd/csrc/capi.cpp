@@ -129,7 +129,8 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
         // (query staging, row table, first tile, writing the partial results: about five and a half tiles' time;
         // three when nothing is split); the merge launch costs about a tile plus a tile per hundred partial rows.
         // Filling every XCD exactly once wins where the batch allows it; a batch that does not divide the CUs
-        // gets fewer, longer splits rather than a second round that is nearly empty.  A split shorter than four
+        // gets fewer, longer splits rather than a second round that is nearly empty, and a batch that needs more
+        // than one round anyway is not split.  A split shorter than four
         // tiles is all prologue.
         // (a size query on a host without a device plans for the 256 CUs of an MI355X; a launch there fails)
         const int cus = cu_count() > 0 ? cu_count() : 256;
@@ -139,6 +140,7 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
         double best = -1.0;
         for (int s = 1; s <= max_split; ++s) {
             const long long rounds = (xcd_rows * pl.hgroups * s + xcd_cus - 1) / xcd_cus;
+            if (rounds > 1 && s > 1) break;              // splitting is for launches that do not fill the chip
             const double merge = s == 1 ? 0.0 : 1.0 + 0.01 * (double)rows * s * pl.hgroups;
             const double cost = (double)rounds * ((tiles + s - 1) / s + (s == 1 ? 3.0 : 5.5)) + merge;
             if (best < 0.0 || cost < best) {
