@@ -6,7 +6,8 @@ A step is one pass of sparse flash attention over one batch: B=32 sequences, one
 scales, per-sequence KV lengths drawn from 8192..65536.  All inputs are resident in HBM before the
 timed region.  Prints ONE JSON line:
 
-  value          query tokens per second (B / step time) over K timed steps
+  value          query tokens per second (B / step time) over K timed steps, after SETTLE_STEPS untimed steps
+                 ("ms_per_step_unsettled": the same K steps timed before them, after the caller's warm-up only)
   roofline       achieved bf16 matrix throughput of the attention launch = algorithmic flops per step
                  / average launch duration from HIP events on the launch stream, against 2.5 PFLOP/s;
                  the HBM-side figure (algorithmic bytes / same duration, against 8 TB/s) is in
@@ -18,9 +19,10 @@ timed region.  Prints ONE JSON line:
   indexer_prolog time of one lightning-indexer prolog pass (projection stage) on the reference's enabled
                  case b=4, s1=2 (8 tokens, h=7168, q_lora_rank=1536), launches replayed from a HIP graph so
                  that host time between launches is not counted, with its HBM fraction
-  mla_prolog     the same for the MLA prolog (b=4, s=2, 128 heads; 85 MB of weights per pass, ten sets)
+  mla_prolog     the same for the MLA prolog (b=4, s=2, 128 heads; 85 MB of weights per pass, ten sets);
+                 all three prolog legs also carry "batch_of_32": the same pass at the headline's 32 tokens
   cpu_baseline   the scalar C statement of the golden, all host threads, on a bounded sample of the
-                 same batch
+                 same batch; beside it the torch golden at configs[0] in its literal loop form and vectorised
 
 To keep a step from being served out of the 256 MB memory-side cache, steps rotate over ROT
 different selections (different indexer queries over the same caches).
@@ -446,6 +448,20 @@ def main():
     # 20 steps take 41.1-42.0 us each after 5 or 255 earlier steps and 38.5-39.1 us after 1000 or 4000.  A
     # decode loop runs for seconds, so the step is timed at the settled clocks whatever --warmup says:
     # SETTLE_STEPS untimed steps come before the warm-up steps (reported as "settle_steps").
+    # The same measurement is taken first with the caller's warm-up alone ("ms_per_step_unsettled"), so that a
+    # change of the kernels and a change of the clocks cannot be mistaken for one another between runs.
+    for i in range(args.warmup):
+        sfa_step(i)
+    torch.cuda.synchronize()
+    evu0, evu1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    tu0 = time.perf_counter()
+    evu0.record()
+    for i in range(args.steps):
+        sfa_step(i)
+    evu1.record()
+    torch.cuda.synchronize()
+    ms_per_step_unsettled = (time.perf_counter() - tu0) / args.steps * 1e3
+    ev_avg_ms_unsettled = evu0.elapsed_time(evu1) / args.steps
     for i in range(SETTLE_STEPS):
         sfa_step(i)
     for i in range(args.warmup):
@@ -476,6 +492,7 @@ def main():
     ws_bytes = C.sfa_quant_workspace_bytes(B, S1, NQ, 1, K, 128, int(sfa_d.block_table.shape[1]), int(sfa_d.key_nope_2d.shape[0]),
                                            float(sfa.softmax_scale), 0)
     key_splits = max(ws_bytes // (B * S1 * NQ * (512 * 2 + 8)), 1)
+    combine_ns = 2 if key_splits <= 2 else (4 if key_splits <= 4 else 8)      # splits the merge kernel holds in flight
     achieved_tflops = flops / (ev_avg_ms * 1e-3) / 1e12
     achieved_gbs = byt / (ev_avg_ms * 1e-3) / 1e9
 
@@ -540,6 +557,9 @@ def main():
     prolog = side_leg(prolog_leg)
     mla_prolog = side_leg(mla_prolog_leg)
     fused_prolog = side_leg(fused_prolog_leg)
+    # ... and at the batch of the headline workload (32 sequences, one token each), fewer weight sets per graph
+    for leg, fn, calls in ((prolog, prolog_leg, 20), (mla_prolog, mla_prolog_leg, 6), (fused_prolog, fused_prolog_leg, 6)):
+        leg["batch_of_32"] = side_leg(lambda t_, d_, p_, fn=fn, calls=calls: fn(t_, d_, p_, b=B, s1=1, calls=calls))
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
@@ -560,6 +580,24 @@ def main():
         cpu = {"value": reps * B / t_cpu, "unit": "tokens/s", "cores": nthreads, "kind": "port",
                "sample": f"the same batch of {B} sequences, {reps} passes of the scalar C golden (OpenMP over "
                          f"heads), {t_cpu:.1f} s"}
+        # configs[0] (B=1, 16 heads, top-k 256, the reference's own CPU-sized case) in the golden's literal form --
+        # one Python iteration per selected key, as the reference gathers them
+        # (deepseekv32_sparse_flash_attention_quant.py:215-228) -- and in the vectorised torch form of the same golden
+        from oracle import sfa_oracle
+        c0 = gen_sfa_inputs(1, 1, 16, config_lengths(0), topk=256, seed=0, shuffle_table=False)
+        a0 = (c0.q_bsnd(), c0.key_nope_2d, c0.key_rope_2d, c0.k_nope_scales, c0.topk_indices, c0.block_table,
+              c0.actual_seq, c0.block_size, c0.softmax_scale, c0.topk)
+        forms = {}
+        for name, fn in (("loop_form", sfa_oracle.sfa_literal_loops), ("vectorised", sfa_oracle.sfa_single_pass)):
+            fn(*a0)
+            n0, t0c = 0, 0.0
+            while t0c < 1.0 and n0 < 2000:
+                tc = time.perf_counter()
+                fn(*a0)
+                t0c += time.perf_counter() - tc
+                n0 += 1
+            forms[name] = {"tokens_per_s": n0 / t0c, "ms_per_call": t0c / n0 * 1e3, "calls": n0}
+        cpu["configs[0]_torch_golden"] = {"workload": "configs[0]: B=1 S_q=1 16 heads topk=256 KV 4096", "torch_threads": torch.get_num_threads(), **forms}
 
     line = {
         "metric": "sfa_decode_tokens_per_s",
@@ -570,6 +608,7 @@ def main():
         "warmup": args.warmup,
         "settle_steps": SETTLE_STEPS,
         "ms_per_step": ms_per_step,
+        "ms_per_step_unsettled": ms_per_step_unsettled,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -583,8 +622,10 @@ def main():
                      "frac": achieved_tflops / PEAK_BF16_TFLOPS,
                      "traffic": measured_traffic(TRAFFIC_FILE, "traffic_bytes_per_step", lib_version,
                                                  {"key_splits": key_splits}),
-                     "kernel": "sfa_decode_kernel<4> + sfa_combine_kernel<8> (one step)",
-                     "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "flops_per_launch": flops},
+                     "kernel": "sfa_decode_kernel<4>" + (f" + sfa_combine_kernel<{combine_ns}>" if key_splits > 1 else "") + " (one step)",
+                     "key_splits": int(key_splits),
+                     "launch_ms_avg": ev_avg_ms, "launch_ms_min": ev_min_ms, "launch_ms_avg_unsettled": ev_avg_ms_unsettled,
+                     "frac_unsettled": flops / (ev_avg_ms_unsettled * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "flops_per_launch": flops},
         "roofline_hbm": {"bound": "hbm", "achieved": achieved_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": achieved_gbs / PEAK_HBM_GBS, "bytes_per_launch": byt},
         "packed_cache": {"operator": "sparse_attention_antiquant_d", "us_per_step": packed_avg_ms * 1e3,

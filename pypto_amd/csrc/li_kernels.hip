@@ -11,18 +11,20 @@
 //
 // Kernels
 //   li_score_kernel   w_scale[h] = fp16(q_scale * weight) if both fp16, else the fp32 product;
-//                     one wave per run of 64-key pairs of blocks: v_mfma_i32_32x32x32_i8 with A = the
-//                     token's 64 query heads (two 32-row operands resident in registers) and
-//                     B = 32 key rows loaded straight from the paged cache in operand layout; a
-//                     half-wave swap gives every lane all 64 heads of one key, summed in registers
-//                     with the per-head factors in scalar registers; scores to a [T, max_seq] fp32
-//                     workspace
+//                     one wave per run of 64-key pairs of blocks: the key rows travel from the paged
+//                     cache into the wave's own LDS buffers by LDS-DMA (whole cache lines, two pairs
+//                     ahead), v_mfma_i32_32x32x32_i8 with A = the token's 64 query heads (two 32-row
+//                     operands resident in registers) and B = 32 key rows read from LDS in operand
+//                     layout; a half-wave swap gives every lane all 64 heads of one key, summed in
+//                     registers with the per-head factors in scalar registers; scores to a
+//                     [T, max_seq] fp32 workspace, and one score of every 16 positions to a compact
+//                     sample array behind it
 //   li_select_kernel  one workgroup per query token, keys ordered by the strict word
-//                     (score image << 32 | ~position): a histogram of a 2048-score sample gives a
-//                     pivot, one pass over the row compacts the keys above it, those are spread over
-//                     2048 buckets linear in the score and ordered inside buckets by counting;
-//                     select_streaming (radix select over the row in memory + bitonic sort) is the
-//                     capacity-free form it falls back to
+//                     (score image << 32 | ~position): a histogram of up to 4096 sampled scores (the
+//                     compact array the score kernel left) gives a pivot, one pass over the row
+//                     compacts the keys above it, those are spread over 2048 buckets linear in the
+//                     score and ordered inside buckets by counting; select_streaming (radix select
+//                     over the row in memory + bitonic sort) is the capacity-free form it falls back to
 #include <type_traits>
 
 #include "common.h"

@@ -31,6 +31,8 @@
 //   mlap_xlinear_mfma_kernel   the sums over the hidden axis on the matrix cores (xlinear_mfma.h) unless the fixed
 //                        order is asked for: per workgroup a 128-column slab x 128 tokens x a range of the hidden
 //                        axis, v_mfma_f32_32x32x16_bf16 with the row-major weight chunk as the transposed operand.
+//   mlap_xlinear_rope_kernel   beside it, the 64 rope columns of w_dkv_kr in their fixed order (the rotated key
+//                        allows no outlier under the reference's acceptance rule).
 //   qproj_prefill_kernel, qproj_prefill256_kernel   the projection unsplit (prolog_common.h), a workgroup per
 //                        128 x 128 or 256 x 256 tile over the whole reduction axis; results leave de-quantised.
 //   mlap_finish_prefill_kernel   per (head, run of 32-token blocks): the head's whole w_uk staged once
@@ -128,6 +130,26 @@ __global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams
     xm_body(sl, p.x, p.T, p.h, t0, (int)((long long)sp * nchunks / nsplit), (int)((long long)(sp + 1) * nchunks / nsplit), smem);
 }
 
+// The 64 rope columns of w_dkv_kr beside the matrix-core form: their sums keep the fixed order at every size
+// (xlinear_fixed.h, the form that broadcasts the hidden states through DPP; workgroup = (group of eight blocks, 16
+// tokens)).  The reference's acceptance rule allows the rotated key no outlier at all
+// (deepseekv32_mla_prolog_quant.py:688: atol 1e-4, rtol 2^-7 per element, ratio 0), and a sum that lands next to a
+// bf16 rounding boundary in another order moves a small rotated value by more than that.
+__global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_rope_kernel(const MlapParams p, const int ngroups)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XD_LDS];
+    const int g = blockIdx.x % ngroups;
+    const int t0 = (blockIdx.x / ngroups) * XD_TOK;
+    const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
+    XlSlab sl;
+    sl.w = reinterpret_cast<const uint8_t *>(p.w_dkvkr) + MLAP_KV * 2;
+    sl.pitch = (MLAP_KV + MLAP_ROPE) * 2;
+    sl.wbytes = MLAP_ROPE * 2;
+    sl.out = p.xpart + (size_t)g * p.T * nc + p.q_lora + MLAP_KV;
+    sl.out_pitch = nc;
+    xd_body<false>(sl, p.x, p.T, p.h, g, t0, smem);
+}
+
 // ---------------------------------------------------------------------------------------------
 constexpr int MID_WAVES = MLAP_MAX_QLORA / 128;   // 12
 
@@ -139,7 +161,9 @@ __device__ __forceinline__ float slab_square_sum(const float v0, const float v1,
 
 // Workgroup 2t: the query latent of token t (one wave per slab of 128 channels).  Workgroup 2t+1: its
 // key latent (waves 0..3) and key rope part (wave 4).
-__global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapParams p, const int ngroups)
+// ngroups partial sums over the hidden axis per column, ngroups_rope for the 64 rope columns (which keep the fixed-order
+// form's groups when the other columns come from the matrix cores).
+__global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapParams p, const int ngroups_other, const int ngroups_rope)
 {
     __shared__ float slabsum[MID_WAVES];
     __shared__ float slabmax[MID_WAVES];
@@ -152,6 +176,7 @@ __global__ __launch_bounds__(64 * MID_WAVES) void mlap_mid_kernel(const MlapPara
     const int nslab = kvtype ? 4 : qslabs;                               // slabs under the norm
     const bool rope_wave = kvtype && w == 4;
     const bool active = w < nslab || rope_wave;
+    const int ngroups = rope_wave ? ngroups_rope : ngroups_other;
     const int col = (kvtype ? p.q_lora : 0) + w * 128 + 2 * (rope_wave ? (l & 31) : l);
 
     // Everything the chain below needs from memory is requested before the first value is looked at: the
@@ -341,6 +366,7 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
 {
     const int nblk = p.h / MLAP_XBLOCK;
     int ngroups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
+    const int ngroups_fixed = ngroups;
     const int nslabs = p.q_lora / 128 + 5;
     if (rider != nullptr && !mlap_takes_rider(p)) return hipErrorInvalidValue;
     const MlapRider rd = rider != nullptr ? *rider : MlapRider{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
@@ -355,9 +381,15 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
         ngroups = ngroups < 1 ? 1 : ngroups;
         ngroups = ngroups > MLAP_XM_MAX_SPLITS ? MLAP_XM_MAX_SPLITS : ngroups;
         ngroups = ngroups > nchunks ? nchunks : ngroups;
+        // every slab but the last, the rope columns, which keep their fixed-order sums
+        const int mslabs = nslabs - 1;
         const int per_slab = ngroups * ttiles;
-        const int wgs = 8 * ((nslabs >> 3) * per_slab + ((nslabs & 7) * per_slab + 7) / 8);   // the kernel's XCD-wise job order
-        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p, nslabs, ngroups);
+        const int wgs = 8 * ((mslabs >> 3) * per_slab + ((mslabs & 7) * per_slab + 7) / 8);   // the kernel's XCD-wise job order
+        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p, mslabs, ngroups);
+        hipError_t e0 = hipGetLastError();
+        if (e0 != hipSuccess) return e0;
+        hipLaunchKernelGGL(mlap_xlinear_rope_kernel, dim3((unsigned)(ngroups_fixed * ((p.T + XD_TOK - 1) / XD_TOK))), dim3(64 * XL_WAVES), 0,
+                           stream, p, ngroups_fixed);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
         const int xslabs = nslabs + (rider != nullptr ? 1 : 0);
@@ -365,7 +397,7 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(mlap_mid_kernel, dim3((unsigned)(2 * p.T)), dim3(64 * MID_WAVES), 0, stream, p, ngroups);
+    hipLaunchKernelGGL(mlap_mid_kernel, dim3((unsigned)(2 * p.T)), dim3(64 * MID_WAVES), 0, stream, p, ngroups, ngroups_fixed);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     const QProj qp = {p.q_norm, p.w_uqqr, p.qpart, p.T, p.q_lora, p.n_heads * MLAP_QHEAD / 128, p.q_norm_scale, p.w_qb_scale};

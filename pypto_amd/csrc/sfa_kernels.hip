@@ -828,12 +828,55 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
 
 // Merges the key splits of one query row: out = sum_s w_s O_s / sum_s w_s with w_s = l_s 2^(m_s - m)
 // and O_s the split's normalised fp16 partial (all zeros for an empty split, whose weight is zero).
-// One thread per (row, head, 8 value channels); splits are taken NS at a time with all their loads in flight
-// together (NS = 2, 4 or 8: the smallest that covers the launch's splits in one trip, so that a row of two
-// splits does not load its last split seven times over).
+// One wave per (row, head), a lane per 8 value channels.  The (max, sum) pairs of a (row, head) are the
+// same for the whole wave and travel through the scalar cache; the NS 16-byte loads of a lane's partials
+// are all requested before the first of them is used.  The kernel moves bytes that were written
+// microseconds earlier, and what it costs is launch and latency, not arithmetic: measured, more and
+// smaller waves are faster than fewer waves with more loads each (2 or 4 (row, head) pairs per wave:
+// 8.2 and 10.2 us against 7.0 at 32 rows x 8 splits).  NS = 2, 4 or 8 splits are in flight at a time:
+// the smallest that covers the launch's splits.
 template <int NS>
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
 {
+    const int lane = threadIdx.x & 63;
+    const int th = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));      // (row, head)
+    if (th >= p.T * p.NQ) return;
+    const int t = th / p.NQ, head = th - t * p.NQ;
+    const size_t prow0 = (size_t)t * p.nsplit * p.NQ + head;       // split s: prow0 + s * NQ
+    const f32x2 *ml = reinterpret_cast<const f32x2 *>(p.part_ml);
+    f16x8 hv[NS];
+    f32x2 v[NS];
+#pragma unroll
+    for (int e = 0; e < NS; ++e) {
+        const size_t prow = prow0 + (size_t)(e < p.nsplit ? e : p.nsplit - 1) * p.NQ;
+        v[e] = ml[prow];
+        hv[e] = *reinterpret_cast<const f16x8 *>(p.part_o + prow * DN + 8 * lane);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < NS; ++e)
+        if (e < p.nsplit && v[e][1] > 0.f) m = fmaxf(m, v[e][0]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float wsum = 0.f;
+#pragma unroll
+    for (int e = 0; e < NS; ++e) {
+        const bool live = e < p.nsplit && v[e][1] > 0.f;
+        const float wgt = live ? v[e][1] * __builtin_amdgcn_exp2f(v[e][0] - m) : 0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[c] += wgt * (float)hv[e][c];
+        wsum += wgt;
+    }
+    const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+    u32x4 outv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) outv[e] = pack_bf16x2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
+    *reinterpret_cast<u32x4 *>(p.out + (size_t)th * DN + 8 * lane) = outv;
+}
+
+// The same merge for any number of splits, eight at a time (rows with more than eight key splits).
+__global__ __launch_bounds__(256) void sfa_combine_many_kernel(const SfaParams p)
+{
+    constexpr int NS = 8;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t total = (size_t)p.T * p.NQ * (DN / 8);
     if (gid >= total) return;
@@ -902,11 +945,17 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.nsplit > 1) {
-        const size_t total = (size_t)p.T * p.NQ * (DN / 8);
-        const dim3 cgrid((unsigned)((total + 255) / 256));
-        if (p.nsplit <= 2) hipLaunchKernelGGL(sfa_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
-        else if (p.nsplit <= 4) hipLaunchKernelGGL(sfa_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
-        else hipLaunchKernelGGL(sfa_combine_kernel<8>, cgrid, dim3(256), 0, stream, p);
+        const int n_th = p.T * p.NQ;
+        if (p.nsplit > 8) {
+            const size_t total = (size_t)n_th * (DN / 8);
+            hipLaunchKernelGGL(sfa_combine_many_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
+        } else {
+            // one wave per (row, head), four waves per workgroup
+            const dim3 cgrid((unsigned)((n_th + 3) / 4));
+            if (p.nsplit <= 2) hipLaunchKernelGGL(sfa_combine_kernel<2>, cgrid, dim3(256), 0, stream, p);
+            else if (p.nsplit <= 4) hipLaunchKernelGGL(sfa_combine_kernel<4>, cgrid, dim3(256), 0, stream, p);
+            else hipLaunchKernelGGL(sfa_combine_kernel<8>, cgrid, dim3(256), 0, stream, p);
+        }
         e = hipGetLastError();
     }
     return e;

@@ -40,6 +40,34 @@ def check(out, ref, what):
     assert max_abs <= MAX_ABS and mean_rel <= MEAN_REL, (what, max_abs, mean_rel)
 
 
+def assert_close_to_fp64_truth(out, gold, inp, rows, what, topk_indices=None):
+    """The sharper bar at full size.  At top-k 2048 an output element is a softmax-weighted mean of 2048 values and
+    about 0.03 in magnitude, so the max-abs bound of 2e-2 says little there.  For a sample of query rows (b, s1)
+    the exact attention -- fp64 scores, softmax and weighted sum over the same de-quantised bf16 keys the golden
+    uses -- is formed, and the kernel's mean-rel error against it may exceed the single-pass golden's own error
+    (its bf16 probabilities and bf16 result) by a quarter at most."""
+    from oracle import sfa_oracle as so
+    ti = inp.topk_indices if topk_indices is None else topk_indices
+    ti = ti.reshape(inp.b * inp.s1, -1).long()
+    num_k = den = num_g = 0.0
+    for b, s1 in rows:
+        cur = min(max(int(inp.actual_seq[b]) - inp.s1 + 1 + s1, 0), inp.topk)
+        assert cur > 0, "sample rows must see keys"
+        idx = ti[b * inp.s1 + s1, :cur]
+        phys = inp.block_table[b].long()[idx // inp.block_size] * inp.block_size + idx % inp.block_size
+        kn = so.dequant_kn(inp.key_nope_2d[phys], inp.k_nope_scales[phys]).double()
+        k = torch.cat([kn, inp.key_rope_2d[phys].double()], dim=-1)
+        q = inp.q_bsnd()[b, s1].double()                                    # [heads, 576]
+        p = torch.softmax((q @ k.T) * inp.softmax_scale, dim=-1)
+        truth = p @ kn                                                      # [heads, 512]
+        num_k += float((out[b, s1].double() - truth).abs().sum())
+        num_g += float((gold[b, s1].double() - truth).abs().sum())
+        den += float(truth.abs().sum())
+    err_k, err_g = num_k / den, num_g / den
+    print(f"{what}: mean-rel error vs fp64 over {len(rows)} rows: kernel {err_k:.4g}, single-pass golden {err_g:.4g}", flush=True)
+    assert err_k <= 1.25 * err_g + 1e-4, (what, err_k, err_g)
+
+
 def test_config2_chain_indexer_then_attention(c_oracle):
     """B=32, KV 8192..65536: the indexer's selection must equal the golden's bit for bit, and the attention
     over it must match the golden within tolerance."""
@@ -58,7 +86,9 @@ def test_config2_chain_indexer_then_attention(c_oracle):
     assert torch.equal(got, want), f"{int((got != want).sum())} index mismatches"
     sel = d.topk_res.reshape(B, K).contiguous()
     out = run_sfa(sfa, topk_indices=sel)
-    check(out, golden(c_oracle, sfa, topk_indices=sel.cpu()), "cfg2 chain")
+    gold = golden(c_oracle, sfa, topk_indices=sel.cpu())
+    check(out, gold, "cfg2 chain")
+    assert_close_to_fp64_truth(out, gold, sfa, [(b, 0) for b in (0, 7, 13, 31)], "cfg2 chain", topk_indices=sel.cpu())
 
 
 def test_config3_two_query_tokens_per_sequence(c_oracle):
@@ -66,7 +96,9 @@ def test_config3_two_query_tokens_per_sequence(c_oracle):
     lengths = config_lengths(3, seed=3)
     inp = gen_sfa_inputs(64, 2, 128, lengths, topk=2048, seed=4)
     out = run_sfa(inp)
-    check(out, golden(c_oracle, inp), "cfg3")
+    gold = golden(c_oracle, inp)
+    check(out, gold, "cfg3")
+    assert_close_to_fp64_truth(out, gold, inp, [(0, 0), (0, 1), (21, 1), (63, 0)], "cfg3")
 
 
 def test_config3_chain_indexer_then_attention(c_oracle):
@@ -107,7 +139,10 @@ def test_config4_prefill_4096_tokens(c_oracle):
     v = (inp.key_nope_2d[phys].float().reshape(4, 128) * inp.k_nope_scales[phys].reshape(4, 1)).reshape(512)
     v = v.to(torch.bfloat16)
     assert torch.equal(out[0, 0].view(torch.int16), v.view(torch.int16).expand(128, 512)), "single-key row"
-    check(out, golden(c_oracle, inp), "cfg4")
+    gold = golden(c_oracle, inp)
+    check(out, gold, "cfg4")
+    # rows that see 2, 100 and 2047 keys, the first with all 2048, a late one and the last
+    assert_close_to_fp64_truth(out, gold, inp, [(0, 1), (0, 99), (0, 2046), (0, 2047), (0, 3333), (0, 4095)], "cfg4")
 
 
 def test_prolog_indexer_chain(c_oracle):
