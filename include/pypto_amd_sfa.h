@@ -132,9 +132,12 @@ int pto_sfa_quant_launch(const PtoSfaQuantArgs *args, void *hip_stream);
  * array built into the library (PTO_SFA_STATIC_SCRATCH_BYTES per GPU, held until
  * the process ends) instead of a workspace; args->workspace and workspace_bytes
  * are ignored.  Nothing is allocated or freed; the first call on a device looks
- * the array's device address up.  A shape whose splits need more than the array
- * holds is refused with PTO_E_WORKSPACE (the decode shapes this library is benchmarked on fit: 32
- * rows x 8 splits and 128 rows x 2 splits of 128 heads take 33.8 MB).
+ * the array's device address up.  With num_splits = 0 the library takes the best
+ * split count whose partial results fit the array (the decode shapes this library
+ * is benchmarked on fit as they are: 32 rows x 8 splits and 128 rows x 2 splits of
+ * 128 heads take 33.8 MB).  An explicit num_splits, or a top-k past what one
+ * workgroup holds, whose splits need more than the array holds is refused with
+ * PTO_E_WORKSPACE.
  * All calls on one GPU share the array: calls whose execution may overlap (two
  * streams, two threads) race on it and must use pto_sfa_quant_launch with
  * workspaces of their own instead.  Nothing in the array has to be cleared
@@ -430,6 +433,15 @@ const char *pto_last_error(void);
 
 /* Library version, "major.minor.patch". */
 const char *pto_version(void);
+
+/*
+ * Revision of the argument structs above.  The structs carry no size field and have grown between revisions
+ * (revision 2 added absorb_exact and a reserved word to PtoMlaPrologQuantArgs, revision 1 was library 0.1.0): a
+ * caller built against another revision would hand over structs of another size.  Compare once after loading:
+ * pto_abi_revision() == PTO_ABI_REVISION, else do not call the launch functions of this library.
+ */
+#define PTO_ABI_REVISION 2
+int pto_abi_revision(void);
 
 #ifdef __cplusplus
 }

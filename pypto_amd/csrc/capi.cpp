@@ -112,7 +112,9 @@ int sfa_check(const PtoSfaQuantArgs *a)
     return PTO_OK;
 }
 
-SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
+// max_bytes: most bytes of partial results the caller can hold; the automatic choice (num_splits = 0) then takes the
+// best split count among those that fit (an explicit count is the caller's own business)
+SfaPlan sfa_plan(const PtoSfaQuantArgs *a, const size_t max_bytes = ~(size_t)0)
 {
     SfaPlan pl;
     pl.waves = a->nq > 64 ? 4 : (a->nq > 32 ? 2 : 1);
@@ -129,9 +131,9 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
         // (query staging, row table, first tile, writing the partial results: about five and a half tiles' time;
         // three when nothing is split); the merge launch costs about a tile plus a tile per hundred partial rows.
         // Filling every XCD exactly once wins where the batch allows it; a batch that does not divide the CUs
-        // gets fewer, longer splits rather than a second round that is nearly empty, and a batch that needs more
-        // than one round anyway is not split.  A split shorter than four
-        // tiles is all prologue.
+        // gets fewer, longer splits rather than a second round that is nearly empty, and a batch of more rows
+        // than CUs is split where shorter workgroups fill its last round better (300 rows: three rounds of half
+        // rows instead of two of whole ones).  A split shorter than four tiles is all prologue.
         // (a size query on a host without a device plans for the 256 CUs of an MI355X; a launch there fails)
         const int cus = cu_count() > 0 ? cu_count() : 256;
         const long long xcd_cus = cus / 8 > 0 ? cus / 8 : 1;
@@ -139,8 +141,8 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a)
         const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
         double best = -1.0;
         for (int s = 1; s <= max_split; ++s) {
+            if (s > 1 && s >= min_split && (size_t)rows * s * a->nq * (512 * sizeof(uint16_t) + 2 * sizeof(float)) > max_bytes) break;
             const long long rounds = (xcd_rows * pl.hgroups * s + xcd_cus - 1) / xcd_cus;
-            if (rounds > 1 && s > 1) break;              // splitting is for launches that do not fill the chip
             const double merge = s == 1 ? 0.0 : 1.0 + 0.01 * (double)rows * s * pl.hgroups;
             const double cost = (double)rounds * ((tiles + s - 1) / s + (s == 1 ? 3.0 : 5.5)) + merge;
             if (best < 0.0 || cost < best) {
@@ -195,10 +197,10 @@ PtoSfaQuantArgs unpacked_view(const PtoSaAntiquantArgs *a)
 
 // checked arguments -> kernel parameters -> launch; the cache is given as three (base, row pitch) pairs
 int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const uint8_t *kr, int kr_pitch, const uint8_t *ksc,
-                int ksc_pitch, void *hip_stream, bool kn_bf16 = false)
+                int ksc_pitch, void *hip_stream, bool kn_bf16 = false, const size_t plan_limit = ~(size_t)0)
 {
     if (cu_count() <= 0) return fail(PTO_E_NO_DEVICE, "sfa: no usable device is current");
-    const SfaPlan pl = sfa_plan(a);
+    const SfaPlan pl = sfa_plan(a, plan_limit);
     if (((long long)(a->b * a->s1) + 7) / 8 * 8 * pl.hgroups * pl.nsplit > 0x7fffffffll)
         return fail(PTO_E_INVALID_ARG, "sfa: rows x head groups x key splits exceeds the largest launch");
     {
@@ -351,6 +353,8 @@ const char *pto_last_error(void) { return g_err; }
 
 const char *pto_version(void) { return "0.5.1"; }
 
+int pto_abi_revision(void) { return PTO_ABI_REVISION; }
+
 int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
 {
     if (!bytes) return fail(PTO_E_INVALID_ARG, "sfa: bytes is NULL");
@@ -379,7 +383,7 @@ int pto_sfa_quant_launch_static(const PtoSfaQuantArgs *a, void *hip_stream)
     if (!a->query_nope || !a->query_rope || !a->key_nope_2d || !a->key_rope_2d || !a->k_nope_scales || !a->topk_indices ||
         !a->block_table || !a->kv_act_seqs || !a->attention_out)
         return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
-    const SfaPlan pl = sfa_plan(a);
+    const SfaPlan pl = sfa_plan(a, SFA_STATIC_SCRATCH_BYTES);
     const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
     if (need > SFA_STATIC_SCRATCH_BYTES)
         return fail(PTO_E_WORKSPACE,
@@ -395,7 +399,7 @@ int pto_sfa_quant_launch_static(const PtoSfaQuantArgs *a, void *hip_stream)
     q.workspace = ptr;
     q.workspace_bytes = SFA_STATIC_SCRATCH_BYTES;
     return sfa_enqueue(&q, static_cast<const int8_t *>(a->key_nope_2d), 512, static_cast<const uint8_t *>(a->key_rope_2d), 128,
-                       static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream);
+                       static_cast<const uint8_t *>(a->k_nope_scales), 16, hip_stream, false, SFA_STATIC_SCRATCH_BYTES);
 }
 
 int pto_sfa_bf16kv_launch(const PtoSfaQuantArgs *a, void *hip_stream)

@@ -467,6 +467,9 @@ constexpr int MLAP_FIN_LDS = 4 * FIN_W_BYTES + MLAP_XTOK * MLAP_NOPE * 4 + MLAP_
 // Workgroup (head, half of the 512 output columns, block of 8 tokens); wave w owns output columns
 // colbase + 64w + l.
 // The work of workgroup wg of the last launch (256 threads), in MLAP_FIN_LDS bytes of LDS at lds.
+// workgroup barriers mlap_finish_body passes (every thread, unconditionally): a launch whose workgroups hold more
+// than this body's 256 threads lets the surplus waves pass as many and leave
+constexpr int MLAP_FIN_BARRIERS = 1;
 __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int wg, uint8_t *lds)
 {
     uint8_t *wsl = lds;
@@ -520,7 +523,7 @@ __device__ __forceinline__ void mlap_finish_body(const MlapParams &p, const int 
         }
     }
     VM_WAIT(0);
-    __syncthreads();
+    __syncthreads();                                   // (counted in MLAP_FIN_BARRIERS)
 
     if (!p.absorb_exact) {
         // On the matrix cores: C^T[col][token] = sum_i W^T[col][i] a^T[i][token], v_mfma_f32_32x32x16_bf16 with

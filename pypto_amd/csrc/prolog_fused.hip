@@ -18,14 +18,17 @@ namespace {
 constexpr int FUSED_FIN_LDS = MLAP_FIN_LDS > LIP_FIN_LDS ? MLAP_FIN_LDS : LIP_FIN_LDS;
 static_assert(2 * FUSED_FIN_LDS <= 160 * 1024, "two workgroups of the last launch share a compute unit");
 
-// Workgroups [0, mla_wgs): the MLA prolog's last launch (its 256 threads; the other four waves leave at once,
-// the barriers of a workgroup count the waves that are still alive).  The rest: the indexer prolog's second launch.
+// Workgroups [0, mla_wgs): the MLA prolog's last launch (its 256 threads; the other four waves pass the body's
+// barriers with them and leave).  The rest: the indexer prolog's second launch.
 __global__ __launch_bounds__(64 * FIN_WAVES) void prolog_fused_finish_kernel(const MlapParams pm, const LipParams pl, const int mla_wgs,
                                                                              const int q_wgs)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lds[FUSED_FIN_LDS];
     if ((int)blockIdx.x < mla_wgs) {
-        if (threadIdx.x >= 256) return;
+        if (threadIdx.x >= 256) {
+            for (int i = 0; i < MLAP_FIN_BARRIERS; ++i) __syncthreads();
+            return;
+        }
         mlap_finish_body(pm, (int)blockIdx.x, lds);
     } else {
         lip_finish_body(pl, q_wgs, (int)blockIdx.x - mla_wgs, lds);

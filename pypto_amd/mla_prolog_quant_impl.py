@@ -3,10 +3,14 @@
 Same callables, argument names and order as ``mla_prolog_quant_d`` / ``mla_prolog_quant_p`` of the reference
 example (examples/models/deepseek_v32_exp/mla_prolog_quant_impl.py:710-869), with the three configuration
 classes its driver fills (:56-94).  ``tile_config`` and ``rope_cfg`` carry NPU tiling hints and are accepted
-and ignored.  Built is the variant of the reference's enabled case
-(deepseekv32_mla_prolog_quant.py:790-834): bf16 ``w_dq`` / ``w_dkv_kr`` (``is_quant_a = False``), int8
-``w_uq_qr`` with per-column ``dequant_scale`` (``is_quant_b = True``), no smoothing, ``cache_mode = "PA_BSND"``;
-anything else raises.  The weight matrices are taken row-major where the reference driver passes their NPU
+and ignored.  Built is what these entry points can reach in the reference, the variant of its enabled case
+(deepseekv32_mla_prolog_quant.py:790-834): bf16 ``w_dq`` / ``w_dkv_kr``, int8 ``w_uq_qr`` with per-column
+``dequant_scale`` (``is_quant_b``), no smoothing.  The reference's ``pre_compute_2d`` also holds branches for int8
+down-projections (``is_quant_a``) and a smoothing factor (:413-458, 479-494), but the entry points build their
+``MlaQuantInputs()`` themselves and fill in ``dequant_scale_w_uq_qr`` only (:609-614): no argument of
+``mla_prolog_quant_d`` / ``_p`` carries the tensors those branches need, and with ``dequant_scale = None`` the
+reference fails at ``q_kv[3]`` (:633), so neither has a caller.  ``cache_mode`` is "PA_BSND" or "PA_NZ" as in the
+reference, which asserts the value (:591) and does the same for both; anything else raises.  The weight matrices are taken row-major where the reference driver passes their NPU
 fractal re-layout (:587-595).  ``k_scale_cache`` is fp32 ``[block_num, block_size, 1, 4]``, the layout the
 sparse attention reads.
 
@@ -95,8 +99,8 @@ def _mla_prolog_quant(token_x, w_dq, w_uq_qr, dequant_scale, w_uk, w_dkv_kr, gam
                       kv_cache_out, kr_cache_out, k_scale_cache_out, epsilon_cq, epsilon_ckv, cache_mode, tile_config,
                       rope_cfg, _collect=None):
     C = _native.load()
-    if cache_mode != "PA_BSND":
-        raise ValueError(f"mla_prolog_quant: cache_mode {cache_mode!r} is not built (only 'PA_BSND')")
+    if cache_mode not in ("PA_BSND", "PA_NZ"):      # the reference asserts the same two and treats them alike (:591)
+        raise ValueError(f"mla_prolog_quant: cache_mode must be 'PA_BSND' or 'PA_NZ', got {cache_mode!r}")
     if dequant_scale is None:
         raise ValueError("mla_prolog_quant: dequant_scale is None (the non-quantized w_uq_qr variant is not built)")
     names = ("token_x", "w_dq", "w_uq_qr", "dequant_scale", "w_uk", "w_dkv_kr", "gamma_cq", "gamma_ckv", "cos", "sin",

@@ -40,6 +40,9 @@ def test_version_and_error_string(lib):
     lib.pto_version.restype = ctypes.c_char_p
     lib.pto_last_error.restype = ctypes.c_char_p
     assert re.fullmatch(rb"\d+\.\d+\.\d+", lib.pto_version())
+    # the revision of the argument structs the library was built with is the one the header states
+    declared = int(re.search(r"#define\s+PTO_ABI_REVISION\s+(\d+)", open(HEADER).read()).group(1))
+    assert lib.pto_abi_revision() == declared
     n = ctypes.c_size_t(0)
     assert lib.pto_sfa_quant_workspace_bytes(None, ctypes.byref(n)) == -1
     assert b"NULL" in lib.pto_last_error()
@@ -128,8 +131,10 @@ def test_prolog_operators_refuse_cpu_tensors_and_unbuilt_variants():
              torch.zeros(1, 2, 64, dtype=torch.bfloat16), mla.kv_cache, mla.kr_cache, mla.k_scale_cache)
     with pytest.raises(RuntimeError):
         pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "PA_BSND", None, None)
+    with pytest.raises(RuntimeError):                    # an accepted cache mode (the reference asserts "PA_BSND" or "PA_NZ"
+        pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "PA_NZ", None, None)   # and treats them alike)
     with pytest.raises(ValueError):
-        pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "PA_NZ", None, None)
+        pypto_amd.mla_prolog_quant_d(*mla.input_tensors(), *mouts, 1e-5, 1e-5, "BSND", None, None)
     args = list(mla.input_tensors())
     args[3] = None                                       # no dequant scale: the non-quantized up-projection
     with pytest.raises(ValueError):

@@ -145,6 +145,19 @@ def test_config4_prefill_4096_tokens(c_oracle):
     assert_close_to_fp64_truth(out, gold, inp, [(0, 1), (0, 99), (0, 2046), (0, 2047), (0, 3333), (0, 4095)], "cfg4")
 
 
+@pytest.mark.parametrize("b,s1", [(300, 1), (128, 4)])
+def test_more_query_rows_than_compute_units(c_oracle, b, s1):
+    """Decode batches past one workgroup per compute unit (the operator's documented range reaches b = 128 with
+    s1 = 4, examples/models/deepseek_v32_exp/README.md:6-24): 300 rows, which the library splits so that the last
+    round of workgroups is not nearly empty, and 512 rows; every row against the golden."""
+    act = [2048 + 37 * (i % 11) for i in range(b)]
+    inp = gen_sfa_inputs(b, s1, 128, act, topk=2048, seed=b + s1)
+    out = run_sfa(inp)
+    gold = golden(c_oracle, inp)
+    check(out, gold, f"b={b} s1={s1}")
+    assert_close_to_fp64_truth(out, gold, inp, [(0, 0), (b // 2, s1 - 1), (b - 1, 0)], f"b={b} s1={s1}")
+
+
 def test_prolog_indexer_chain(c_oracle):
     """Prolog -> indexer on the GPU against prolog oracle -> indexer oracle: the prolog's int8 query, fp16 scales
     and weights and its freshly written key rows feed the indexer; the selected indices must be identical."""

@@ -135,6 +135,22 @@ def test_token_pairs_share_a_key_pass(c_oracle, variant, b, s1):
     assert_exact(run_op(inp), oracle(inp, c_oracle), f"{variant} b={b} s1={s1}")
 
 
+@pytest.mark.parametrize("variant,b,s1", [("fp16", 260, 4), ("fp32", 260, 3)])
+def test_token_pairs_beyond_the_balanced_mapping(c_oracle, variant, b, s1):
+    """Token pairs per key pass in the launch shape that takes one grid row per unit: more than 512 units (260
+    sequences of two units each) with enough keys for the pair form -- the far end of the operator's documented
+    decode range (b up to 128 with s1 up to 4 and long KV, examples/models/deepseek_v32_exp/README.md:6-24, and
+    past it).  The odd s1 leaves every sequence a unit of one token."""
+    g = torch.Generator().manual_seed(500 + s1)
+    act = [int(x) for x in torch.randint(s1, 2300, [b], generator=g)]
+    act[0], act[1], act[-1] = 2300, 2049, s1
+    inp = gen_indexer_inputs(b, s1, act, selected_count=2048, seed=b + s1, variant=variant)
+    units = inp.b * ((s1 + 1) // 2)
+    assert units > 512, "shape must be past the balanced mapping"
+    assert units * (inp.block_table.shape[1] * 128 // 64) >= 8 * 256 * 8, "shape too small for token pairs"
+    assert_exact(run_op(inp), oracle(inp, c_oracle), f"{variant} b={b} s1={s1}")
+
+
 def test_small_pages_and_small_k(c_oracle):
     """32-key pages (every block of a pair on its own page) and small selection counts."""
     for k, act in ((1, [5000, 70]), (17, [2500, 31]), (512, [700, 513])):

@@ -26,7 +26,7 @@ def exact_absorb():
     impl.EXACT_ABSORB, lip_impl.EXACT_SUMS, lip_impl.MATRIX_CORE_HIDDEN_SUMS = old
 
 
-def run_op(inp, eps=(0.0, 0.0), separate_cache_out=False, prefill=False):
+def run_op(inp, eps=(0.0, 0.0), separate_cache_out=False, prefill=False, cache_mode="PA_BSND"):
     dev = torch.device("cuda:0")
     d = inp.to(dev)
     t, n, ql = d.token_x.shape[0], d.w_uk.shape[0], d.w_dq.shape[1]
@@ -41,7 +41,7 @@ def run_op(inp, eps=(0.0, 0.0), separate_cache_out=False, prefill=False):
     ins = [pypto_amd.from_torch(v) for v in d.input_tensors()]
     outs = [pypto_amd.from_torch(v) for v in (q_norm, q_norm_scale, q_nope, q_rope, kv, kr, ks)]
     fn = pypto_amd.mla_prolog_quant_p if prefill else pypto_amd.mla_prolog_quant_d
-    ret = fn(*ins, *outs, eps[0], eps[1], "PA_BSND", pypto_amd.MlaTileConfig(), pypto_amd.RopeTileShapeConfig())
+    ret = fn(*ins, *outs, eps[0], eps[1], cache_mode, pypto_amd.MlaTileConfig(), pypto_amd.RopeTileShapeConfig())
     assert ret is None
     torch.cuda.synchronize()
     return {"q_norm": q_norm.cpu().numpy(), "q_norm_scale": q_norm_scale.cpu().numpy()[:, 0],
@@ -93,6 +93,14 @@ def test_mla_prolog_small_shapes_bit_exact(b, s1, act, kw, eps):
     inp = gen_mla_prolog_inputs(b, s1, act, seed=3 * b + s1, **kw)
     ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=eps[0], epsilon_ckv=eps[1])
     assert_exact(run_op(inp, eps), ref, f"b={b} s1={s1} {kw}")
+
+
+def test_mla_prolog_cache_mode_pa_nz_is_accepted_and_changes_nothing():
+    """The reference asserts cache_mode in ("PA_BSND", "PA_NZ") and does nothing else with it
+    (mla_prolog_quant_impl.py:591): both values give the same outputs and cache rows."""
+    inp = gen_mla_prolog_inputs(2, 2, [300, 129], seed=8, h=256, q_lora_rank=512, n_heads=4)
+    ref = mo.mla_prolog_ref(*inp.input_tensors(), epsilon_cq=1e-5, epsilon_ckv=1e-5)
+    assert_exact(run_op(inp, (1e-5, 1e-5), cache_mode="PA_NZ"), ref, "PA_NZ")
 
 
 def test_mla_prolog_reference_case_b4_s2():
