@@ -91,6 +91,7 @@ struct SfaPlan {
     int waves;
     int hgroups;
     int nsplit;
+    int whole_slots;      // rows 0 .. 8 * whole_slots - 1 are not split
     size_t part_o_bytes;
     size_t part_ml_bytes;
 };
@@ -155,9 +156,41 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a, const size_t max_bytes = ~(size_t)0)
     ns = ns > tiles ? tiles : ns;
     ns = ns < 1 ? 1 : ns;
     pl.nsplit = ns;
-    if (ns > 1) {
-        pl.part_o_bytes = (size_t)rows * ns * a->nq * 512 * sizeof(uint16_t);
-        pl.part_ml_bytes = (size_t)rows * ns * a->nq * 2 * sizeof(float);
+    pl.whole_slots = 0;
+    long long split_rows = rows;
+    if (a->num_splits == 0 && min_split == 1) {
+        // More rows than compute units: the full rounds of whole rows first, then the rows left over dealt out in
+        // as many pieces as fill one more round (300 rows on 256 CUs: 32 whole rows per XCD, the other five or
+        // six in five pieces each), where that beats the best uniform split above.
+        const int cus = cu_count() > 0 ? cu_count() : 256;
+        const long long xcd_cus = cus / 8 > 0 ? cus / 8 : 1;
+        const long long xcd_rows = (rows + 7) / 8;
+        const long long per_round = xcd_cus / pl.hgroups;                 // rows of an XCD that one round holds
+        const long long full = per_round > 0 ? xcd_rows / per_round : 0;
+        const long long rem = per_round > 0 ? xcd_rows - full * per_round : 0;
+        if (full >= 1 && rem >= 1) {
+            int sb = (int)(per_round / rem);
+            const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
+            sb = sb > max_split ? max_split : sb;
+            const long long rows_b = rows - 8 * full * per_round;         // rows 8 * whole_slots and up
+            if (sb >= 2 && rows_b > 0 &&
+                (size_t)rows_b * sb * a->nq * (512 * sizeof(uint16_t) + 2 * sizeof(float)) <= max_bytes) {
+                const double merge = 1.0 + 0.01 * (double)rows_b * sb * pl.hgroups;
+                const double cost = (double)full * (tiles + 3.0) + ((tiles + sb - 1) / sb + 5.5) + merge;
+                const long long rounds_u = (xcd_rows * pl.hgroups * ns + xcd_cus - 1) / xcd_cus;
+                const double cost_u = (double)rounds_u * ((tiles + ns - 1) / ns + (ns == 1 ? 3.0 : 5.5)) +
+                                      (ns == 1 ? 0.0 : 1.0 + 0.01 * (double)rows * ns * pl.hgroups);
+                if (cost < cost_u) {
+                    pl.nsplit = sb;
+                    pl.whole_slots = (int)(full * per_round);
+                    split_rows = rows_b;
+                }
+            }
+        }
+    }
+    if (pl.nsplit > 1) {
+        pl.part_o_bytes = (size_t)split_rows * pl.nsplit * a->nq * 512 * sizeof(uint16_t);
+        pl.part_ml_bytes = (size_t)split_rows * pl.nsplit * a->nq * 2 * sizeof(float);
     } else {
         pl.part_o_bytes = pl.part_ml_bytes = 0;
     }
@@ -201,7 +234,7 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
 {
     if (cu_count() <= 0) return fail(PTO_E_NO_DEVICE, "sfa: no usable device is current");
     const SfaPlan pl = sfa_plan(a, plan_limit);
-    if (((long long)(a->b * a->s1) + 7) / 8 * 8 * pl.hgroups * pl.nsplit > 0x7fffffffll)
+    if (((long long)(a->b * a->s1) + 7) / 8 * 8 * pl.hgroups * pl.nsplit > 0x7fffffffll)     // (an upper bound of the grid)
         return fail(PTO_E_INVALID_ARG, "sfa: rows x head groups x key splits exceeds the largest launch");
     {
         const void *al16[] = {a->query_nope, a->query_rope, kn, kr, ksc, a->attention_out, a->workspace};
@@ -241,6 +274,7 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
     p.bs = (int)a->block_size;
     p.maxblk = (int)a->max_blocknum_perbatch;
     p.nsplit = pl.nsplit;
+    p.whole_slots = pl.whole_slots;
     p.hgroups = pl.hgroups;
     p.waves = pl.waves;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;

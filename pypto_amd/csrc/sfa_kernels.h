@@ -22,11 +22,13 @@ struct SfaParams {
     const int32_t *bt;        // [B, maxblk]
     const int32_t *act;       // [B]
     uint16_t *out;            // [T*NQ, 512] bf16
-    uint16_t *part_o;         // [T, nsplit, NQ, 512] fp16: O / l of each key split (nsplit > 1)
-    float *part_ml;           // [T, nsplit, NQ, 2]   reference max (log2 domain) and row sum of the split
+    uint16_t *part_o;         // [split rows, nsplit, NQ, 512] fp16: O / l of each key split (nsplit > 1)
+    float *part_ml;           // [split rows, nsplit, NQ, 2]   reference max (log2 domain) and row sum of the split
     long long kv_rows;
     int T, S1, NQ, topk, bs, maxblk;
-    int nsplit;               // key splits per query row
+    int nsplit;               // key splits per query row, of the rows that are split
+    int whole_slots;          // rows 0 .. 8 * whole_slots - 1 are not split (one workgroup per row and head group): the
+                              // full rounds of a launch of more rows than compute units; 0 = every row is split alike
     int hgroups;              // head groups per query row (32*waves heads each)
     int waves;                // waves per workgroup: 1, 2 or 4
     float scale_log2;         // softmax_scale * log2(e)

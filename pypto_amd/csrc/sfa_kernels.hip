@@ -162,15 +162,28 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     const int half = l >> 5;
     const int col = l & 31;
 
-    // workgroups of one query row share an XCD (consecutive workgroup ids rotate over the 8 XCDs)
-    const int per_row = p.hgroups * p.nsplit;
+    // Workgroups of one query row share an XCD (consecutive workgroup ids rotate over the 8 XCDs): row t is row
+    // slot t / 8 of XCD t % 8.  The first whole_slots row slots of every XCD are rows taken by one workgroup each
+    // (per head group), the others are split over nsplit workgroups: a launch of more rows than compute units
+    // runs its full rounds of whole rows first and deals the rows left over out in pieces.
     const int xcd = blockIdx.x & 7;
     const int slot = blockIdx.x >> 3;
-    const int t = (slot / per_row) * 8 + xcd;
+    const int wslots = p.whole_slots * p.hgroups;
+    int rslot, within, nsplit;
+    if (slot < wslots) {
+        rslot = slot / p.hgroups;
+        within = slot - rslot * p.hgroups;
+        nsplit = 1;
+    } else {
+        const int per_row = p.hgroups * p.nsplit;
+        rslot = p.whole_slots + (slot - wslots) / per_row;
+        within = (slot - wslots) % per_row;
+        nsplit = p.nsplit;
+    }
+    const int t = rslot * 8 + xcd;
     if (t >= p.T) return;
-    const int within = slot % per_row;
-    const int hg = within / p.nsplit;
-    const int sp = within % p.nsplit;
+    const int hg = within / nsplit;
+    const int sp = within % nsplit;
     const int b = t / p.S1;
     const int s1i = t - b * p.S1;
 
@@ -180,7 +193,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
     // keys [kb, ke) of a row with n selected keys that this split takes
     auto split_keys = [&](const int n, int &kb, int &ke) {
         const int ntile = (n + KT - 1) / KT;
-        const int tiles_per_split = (ntile + p.nsplit - 1) / p.nsplit;
+        const int tiles_per_split = (ntile + nsplit - 1) / nsplit;
         kb = sp * tiles_per_split * KT;
         ke = kb + tiles_per_split * KT;
         ke = ke > n ? n : ke;
@@ -754,7 +767,7 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
         // row-wise reads (two heads, 16 even or odd chunks each) both touch every bank once.
         uint8_t *stage = reinterpret_cast<uint8_t *>(pool) + w * (32 * 256);
         const int head_base = hg * (32 * NW) + w * 32;
-        const size_t prow_base = ((size_t)t * p.nsplit + sp) * p.NQ;
+        const size_t prow_base = ((size_t)(t - 8 * p.whole_slots) * nsplit + sp) * p.NQ;    // split rows only
         const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         // FINAL: bf16 result rows; otherwise fp16 partial of a key split (O / l of the split, merged by
         // the combine kernel with weights l * 2^(m - m_max); O / l is a convex combination of
@@ -812,14 +825,14 @@ __global__ __launch_bounds__(NW * 64) void sfa_decode_kernel(const SfaParams p)
             }
         };
         const bool all_heads = head_base + 32 <= p.NQ;
-        if (p.nsplit == 1) {
+        if (nsplit == 1) {
             if (all_heads) drain(std::true_type{}, std::true_type{});
             else drain(std::true_type{}, std::false_type{});
         } else {
             if (all_heads) drain(std::false_type{}, std::true_type{});
             else drain(std::false_type{}, std::false_type{});
         }
-        if (p.nsplit > 1 && half == 0 && head_ok) {
+        if (nsplit > 1 && half == 0 && head_ok) {
             p.part_ml[(prow_base + head) * 2] = m_run;
             p.part_ml[(prow_base + head) * 2 + 1] = l_run;
         }
@@ -839,10 +852,12 @@ template <int NS>
 __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
 {
     const int lane = threadIdx.x & 63;
-    const int th = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));      // (row, head)
-    if (th >= p.T * p.NQ) return;
-    const int t = th / p.NQ, head = th - t * p.NQ;
-    const size_t prow0 = (size_t)t * p.nsplit * p.NQ + head;       // split s: prow0 + s * NQ
+    // (row, head) among the split rows, which are rows 8 * whole_slots and up
+    const int th = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+    const int t_first = 8 * p.whole_slots;
+    if (th >= (p.T - t_first) * p.NQ) return;
+    const int ts = th / p.NQ, head = th - ts * p.NQ;
+    const size_t prow0 = (size_t)ts * p.nsplit * p.NQ + head;      // split s: prow0 + s * NQ
     const f32x2 *ml = reinterpret_cast<const f32x2 *>(p.part_ml);
     f16x8 hv[NS];
     f32x2 v[NS];
@@ -870,7 +885,7 @@ __global__ __launch_bounds__(256) void sfa_combine_kernel(const SfaParams p)
     u32x4 outv;
 #pragma unroll
     for (int e = 0; e < 4; ++e) outv[e] = pack_bf16x2(acc[2 * e] * inv, acc[2 * e + 1] * inv);
-    *reinterpret_cast<u32x4 *>(p.out + (size_t)th * DN + 8 * lane) = outv;
+    *reinterpret_cast<u32x4 *>(p.out + ((size_t)t_first * p.NQ + th) * DN + 8 * lane) = outv;
 }
 
 // The same merge for any number of splits, eight at a time (rows with more than eight key splits).
@@ -878,13 +893,15 @@ __global__ __launch_bounds__(256) void sfa_combine_many_kernel(const SfaParams p
 {
     constexpr int NS = 8;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t total = (size_t)p.T * p.NQ * (DN / 8);
+    const int t_first = 8 * p.whole_slots;                         // the split rows are rows t_first and up
+    const size_t total = (size_t)(p.T - t_first) * p.NQ * (DN / 8);
     if (gid >= total) return;
     const int c8 = (int)(gid % (DN / 8));
     const size_t th = gid / (DN / 8);
     const int head = (int)(th % p.NQ);
-    const int t = (int)(th / p.NQ);
-    const size_t prow0 = (size_t)t * p.nsplit * p.NQ + head;       // split s: prow0 + s * NQ
+    const int ts = (int)(th / p.NQ);
+    const int t = t_first + ts;
+    const size_t prow0 = (size_t)ts * p.nsplit * p.NQ + head;      // split s: prow0 + s * NQ
     const f32x2 *ml = reinterpret_cast<const f32x2 *>(p.part_ml);
 
     float m = -INFINITY;
@@ -927,8 +944,8 @@ __global__ __launch_bounds__(256) void sfa_combine_many_kernel(const SfaParams p
 
 hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
 {
-    const int rows8 = (p.T + 7) / 8 * 8;
-    const unsigned grid = (unsigned)(rows8 * p.hgroups * p.nsplit);
+    const int rslots = (p.T + 7) / 8;                      // row slots per XCD
+    const unsigned grid = (unsigned)(8 * p.hgroups * (p.whole_slots + (rslots - p.whole_slots) * p.nsplit));
     if (p.kn_bf16) {
         switch (p.waves) {
         case 1: hipLaunchKernelGGL((sfa_decode_kernel<1, false>), dim3(grid), dim3(64), 0, stream, p); break;
@@ -944,8 +961,8 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (p.nsplit > 1) {
-        const int n_th = p.T * p.NQ;
+    if (p.nsplit > 1 && p.T > 8 * p.whole_slots) {
+        const int n_th = (p.T - 8 * p.whole_slots) * p.NQ;
         if (p.nsplit > 8) {
             const size_t total = (size_t)n_th * (DN / 8);
             hipLaunchKernelGGL(sfa_combine_many_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);

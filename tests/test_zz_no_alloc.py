@@ -84,28 +84,18 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     assert b"scratch" in lib.pto_last_error()
 
 
-def test_static_scratch_entry_point_chooses_its_splits_within_the_array():
-    """num_splits = 0 on a launch for which the library's own choice (300 rows: two splits, 79 MB of partial
-    results) exceeds the built-in array: the static entry point takes the best count that fits -- here none, one
-    workgroup per row -- and gives the bits of the workspace entry point told to do the same.  When even the fewest
-    splits a shape allows (top-k past what one workgroup holds) exceed the array, the call is refused."""
+def test_static_scratch_entry_point_with_the_library_s_own_split_choice():
+    """num_splits = 0 on a launch of more rows than compute units (300 rows: the first 256 whole, the other 44 in
+    five pieces each, partial results in the built-in array): the bits of the workspace entry point with the same
+    choice.  When even the fewest splits a shape allows (top-k past what one workgroup holds) exceed the array,
+    the call is refused."""
     lib = ctypes.CDLL(LIB)
     lib.pto_last_error.restype = ctypes.c_char_p
     torch.cuda.synchronize()
     inp = gen_sfa_inputs(300, 1, 128, [2048 + 16 * (i % 5) for i in range(300)], topk=2048, seed=13)
-    need = ctypes.c_size_t(0)
-    dev = torch.device("cuda:0")
-    d = inp.to(dev)
-    out = torch.full([inp.b, inp.s1, inp.n_q, 512], float("nan"), dtype=torch.bfloat16, device=dev)
-    a = _args(d, out, inp, 0)
-    assert lib.pto_sfa_quant_workspace_bytes(ctypes.byref(a), ctypes.byref(need)) == 0
-    assert need.value > (40 << 20), "the shape is meant to want more than the array holds"
-    print(f"static scratch, automatic splits: the unbounded plan wants {need.value} bytes", flush=True)
-    assert lib.pto_sfa_quant_launch_static(ctypes.byref(a), None) == 0, lib.pto_last_error()
-    torch.cuda.synchronize()
-    ws_out, _ = _both(lib, inp, 1)
-    assert not torch.isnan(out).any()
-    assert torch.equal(out.cpu().view(torch.int16), ws_out.view(torch.int16))
+    ws_out, static_out = _both(lib, inp, 0)
+    assert not torch.isnan(static_out).any()
+    assert torch.equal(ws_out.view(torch.int16), static_out.view(torch.int16))
     # top-k 8192 needs four splits at least (2048 keys per workgroup): 128 rows x 4 x 128 heads exceed the array
     forced = PtoSfaQuantArgs()
     for f in ("query_nope", "query_rope", "key_nope_2d", "key_rope_2d", "k_nope_scales", "topk_indices", "block_table",
