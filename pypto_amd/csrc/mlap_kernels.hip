@@ -31,8 +31,8 @@
 //   mlap_xlinear_mfma_kernel   the sums over the hidden axis on the matrix cores (xlinear_mfma.h) unless the fixed
 //                        order is asked for: per workgroup a 128-column slab x 128 tokens x a range of the hidden
 //                        axis, v_mfma_f32_32x32x16_bf16 with the row-major weight chunk as the transposed operand.
-//   mlap_xlinear_rope_kernel   beside it, the 64 rope columns of w_dkv_kr in their fixed order (the rotated key
-//                        allows no outlier under the reference's acceptance rule).
+//                        The launch's first workgroups take the 64 rope columns of w_dkv_kr in their fixed order
+//                        instead (the rotated key allows no outlier under the reference's acceptance rule).
 //   qproj_prefill_kernel, qproj_prefill256_kernel   the projection unsplit (prolog_common.h), a workgroup per
 //                        128 x 128 or 256 x 256 tile over the whole reduction axis; results leave de-quantised.
 //   mlap_finish_prefill_kernel   per (head, run of 32-token blocks): the head's whole w_uk staged once
@@ -95,15 +95,38 @@ __global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_kernel(const MlapP
 // one of nsplit ranges of the hidden axis, 128 tokens); the 64 rope columns are a narrow slab of their own.
 static_assert(XM_KC == MLAP_XBLOCK, "the workspace is sized in chunks of the hidden axis");
 
-__global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams p, const int nslabs, const int nsplit)
+// The first rope_wgs workgroups of the launch (a multiple of eight, so that the XCD-wise order of the others keeps)
+// take the 64 rope columns of w_dkv_kr instead, in their fixed order at every size (xlinear_fixed.h, the four-wave DPP
+// form; workgroup = (group of eight blocks, 16 tokens)): the reference's acceptance rule allows the rotated key no
+// outlier at all (deepseekv32_mla_prolog_quant.py:688: atol 1e-4, rtol 2^-7 per element, ratio 0), and a sum that
+// lands next to a bf16 rounding boundary in another order moves a small rotated value by more than that.
+static_assert(XR_LDS <= XM_LDS, "the rope jobs fit the launch's LDS");
+__global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams p, const int nslabs, const int nsplit, const int rope_wgs,
+                                                                const int rope_groups)
 {
     __shared__ __attribute__((aligned(16))) uint8_t smem[XM_LDS];
+    if ((int)blockIdx.x < rope_wgs) {
+        const int j = blockIdx.x;
+        const int g = j % rope_groups;
+        const int t0 = (j / rope_groups) * XD_TOK;
+        if (t0 >= p.T) return;                         // padding of the count to a multiple of eight
+        const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
+        XlSlab sl;
+        sl.w = reinterpret_cast<const uint8_t *>(p.w_dkvkr) + MLAP_KV * 2;
+        sl.pitch = (MLAP_KV + MLAP_ROPE) * 2;
+        sl.wbytes = MLAP_ROPE * 2;
+        sl.out = p.xpart + (size_t)g * p.T * nc + p.q_lora + MLAP_KV;
+        sl.out_pitch = nc;
+        xr_body(sl, p.x, p.T, p.h, g, t0, smem);
+        return;
+    }
+    const int bid = (int)blockIdx.x - rope_wgs;
     // Workgroups go round the eight XCDs, each with an L2 of its own, and the working set (hidden states + weights)
     // is several times one L2: the jobs of a slab (its ranges of h x token tiles) all run on XCD slab % 8, so a slab's
     // weights cross into one L2 only and every XCD reads the hidden states once for its two or so slabs.  The slabs
     // left over when their number is no multiple of eight are dealt out job by job.
     const int per_slab = nsplit * ((p.T + XM_TOK - 1) / XM_TOK);
-    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int xcd = bid & 7, j = bid >> 3;
     const int full = nslabs >> 3;
     int slab, rem;
     if (j < full * per_slab) {
@@ -128,26 +151,6 @@ __global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams
     sl.out_pitch = nc;
     const int nchunks = p.h / XM_KC;
     xm_body(sl, p.x, p.T, p.h, t0, (int)((long long)sp * nchunks / nsplit), (int)((long long)(sp + 1) * nchunks / nsplit), smem);
-}
-
-// The 64 rope columns of w_dkv_kr beside the matrix-core form: their sums keep the fixed order at every size
-// (xlinear_fixed.h, the form that broadcasts the hidden states through DPP; workgroup = (group of eight blocks, 16
-// tokens)).  The reference's acceptance rule allows the rotated key no outlier at all
-// (deepseekv32_mla_prolog_quant.py:688: atol 1e-4, rtol 2^-7 per element, ratio 0), and a sum that lands next to a
-// bf16 rounding boundary in another order moves a small rotated value by more than that.
-__global__ __launch_bounds__(64 * XL_WAVES) void mlap_xlinear_rope_kernel(const MlapParams p, const int ngroups)
-{
-    __shared__ __attribute__((aligned(16))) uint8_t smem[XD_LDS];
-    const int g = blockIdx.x % ngroups;
-    const int t0 = (blockIdx.x / ngroups) * XD_TOK;
-    const int nc = p.q_lora + MLAP_KV + MLAP_ROPE;
-    XlSlab sl;
-    sl.w = reinterpret_cast<const uint8_t *>(p.w_dkvkr) + MLAP_KV * 2;
-    sl.pitch = (MLAP_KV + MLAP_ROPE) * 2;
-    sl.wbytes = MLAP_ROPE * 2;
-    sl.out = p.xpart + (size_t)g * p.T * nc + p.q_lora + MLAP_KV;
-    sl.out_pitch = nc;
-    xd_body<false>(sl, p.x, p.T, p.h, g, t0, smem);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -385,11 +388,9 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
         const int mslabs = nslabs - 1;
         const int per_slab = ngroups * ttiles;
         const int wgs = 8 * ((mslabs >> 3) * per_slab + ((mslabs & 7) * per_slab + 7) / 8);   // the kernel's XCD-wise job order
-        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p, mslabs, ngroups);
-        hipError_t e0 = hipGetLastError();
-        if (e0 != hipSuccess) return e0;
-        hipLaunchKernelGGL(mlap_xlinear_rope_kernel, dim3((unsigned)(ngroups_fixed * ((p.T + XD_TOK - 1) / XD_TOK))), dim3(64 * XL_WAVES), 0,
-                           stream, p, ngroups_fixed);
+        const int rope_wgs = (ngroups_fixed * ((p.T + XD_TOK - 1) / XD_TOK) + 7) / 8 * 8;
+        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)(rope_wgs + wgs)), dim3(256), 0, stream, p, mslabs, ngroups, rope_wgs,
+                           ngroups_fixed);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
         const int xslabs = nslabs + (rider != nullptr ? 1 : 0);

@@ -289,5 +289,94 @@ __device__ __forceinline__ void xd_body(const XlSlab &sl, const uint16_t *x, con
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The DPP form for a slab of 64 columns in a workgroup of FOUR waves, so that its jobs can ride in a launch whose
+// workgroups have 256 threads: wave w takes blocks w and w + 4 of the group one after the other (the same 64
+// sequential multiply-adds per block from 0.0), the eight block sums are parked in LDS beside the staging areas and
+// chained ascending into the group sum -- product by product and sum by sum what xd_body<false> computes, so the
+// same bits.  LDS: four staging areas of 64 rows x 128 bytes, then eight block-sum areas of [XD_TOK][64] floats.
+constexpr int XR_WAVES = 4;
+constexpr int XR_STAGE = XL_BLOCK * 128;                                 // a block of the slab: 64 rows x 128 bytes
+constexpr int XR_SUMS = XD_TOK * 64 * 4;
+constexpr int XR_LDS = XR_WAVES * XR_STAGE + XL_GROUP * XR_SUMS;
+
+__device__ __forceinline__ void xr_body(const XlSlab &sl, const uint16_t *x, const int T, const int h, const int g, const int t0, uint8_t *smem)
+{
+    const int l = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nblk = h / XL_BLOCK;
+    constexpr int wbytes = 128;
+    uint8_t *region = smem + w * XR_STAGE;
+    const int nb = nblk - g * XL_GROUP < XL_GROUP ? nblk - g * XL_GROUP : XL_GROUP;
+#pragma unroll 1
+    for (int pass = 0; pass < XL_GROUP / XR_WAVES; ++pass) {
+        const int bi = w + XR_WAVES * pass;                               // this wave's block of the group
+        if (bi < nb) {
+            float a0[XD_TOK], a1[XD_TOK];
+#pragma unroll
+            for (int t = 0; t < XD_TOK; ++t) a0[t] = a1[t] = 0.f;
+            const int k0 = (g * XL_GROUP + bi) * XL_BLOCK;
+            const uint32_t wdst = (uint32_t)(uintptr_t)(lds_byte_t *)region;
+            {   // rows of 128 bytes: eight lanes per row, eight rows per request
+                const uint8_t *src = sl.w + (size_t)(k0 + (l >> 3)) * sl.pitch + 16 * (l & 7);
+#pragma unroll 1
+                for (int i = 0; i < XL_BLOCK / 8; ++i) dma16(src + (size_t)i * 8 * sl.pitch, wdst + 1024 * i);
+            }
+            uint32_t xr[2][XD_TOK];
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb)
+#pragma unroll
+                for (int t = 0; t < XD_TOK; ++t) {
+                    const int tt = t0 + t < T ? t0 + t : T - 1;
+                    xr[hb][t] = reinterpret_cast<const uint32_t *>(x + (size_t)tt * h + k0 + 32 * hb)[l & 15];
+                }
+            VM_WAIT(0);
+            const int lane_off = 2 * l;
+#pragma unroll
+            for (int hb = 0; hb < 2; ++hb) {
+                float xe[XD_TOK], xo[XD_TOK];
+#pragma unroll
+                for (int t = 0; t < XD_TOK; ++t) {
+                    xe[t] = __uint_as_float(xr[hb][t] << 16);
+                    xo[t] = __uint_as_float(xr[hb][t] & 0xffff0000u);
+                }
+                const uint8_t *wrow = region + 32 * hb * wbytes;
+                xd_pair_of_rows<false, 0>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 1>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 2>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 3>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 4>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 5>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 6>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 7>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 8>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 9>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 10>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 11>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 12>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 13>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 14>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+                xd_pair_of_rows<false, 15>(wrow, wbytes, lane_off, xe, xo, a0, a1);
+            }
+            // (the LDS reads of the weights above are complete: their results were consumed by the multiply-adds)
+            float *bs = reinterpret_cast<float *>(smem + XR_WAVES * XR_STAGE + bi * XR_SUMS);
+#pragma unroll
+            for (int t = 0; t < XD_TOK; ++t) bs[t * 64 + l] = a0[t];
+        }
+    }
+    __syncthreads();
+    // group sums: wave w chains the block sums of tokens w, w + 4, w + 8, w + 12 in ascending order
+#pragma unroll
+    for (int u = 0; u < XD_TOK / XR_WAVES; ++u) {
+        const int tl = w + XR_WAVES * u;
+        const int t = t0 + tl;
+        if (t < T) {
+            float s0 = 0.f;
+            for (int i = 0; i < nb; ++i) s0 = __fadd_rn(s0, reinterpret_cast<const float *>(smem + XR_WAVES * XR_STAGE + i * XR_SUMS)[tl * 64 + l]);
+            sl.out[(size_t)t * sl.out_pitch + l] = s0;
+        }
+    }
+}
+
 }  // namespace
 }  // namespace pto
