@@ -94,7 +94,11 @@ struct SfaPlan {
     int whole_slots;      // rows 0 .. 8 * whole_slots - 1 are not split
     size_t part_o_bytes;
     size_t part_ml_bytes;
+    size_t predeq_bytes;  // the whole cache de-quantised once, behind the partial results (0: not worth it)
+    size_t predeq_offset; // where in the workspace
 };
+
+constexpr size_t SFA_PREDEQ_MAX_BYTES = (size_t)64 << 20;
 
 int sfa_check(const PtoSfaQuantArgs *a)
 {
@@ -194,8 +198,18 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a, const size_t max_bytes = ~(size_t)0)
     } else {
         pl.part_o_bytes = pl.part_ml_bytes = 0;
     }
+    // A launch that selects every cache row many times over (a prefill chunk: thousands of query rows over a few
+    // thousand keys) de-quantises the cache once into the workspace and attends over the bf16 rows -- the same
+    // bits, since the kernel's bf16-cache form reads exactly what its int8 form converts to, without the per-tile
+    // conversion (8 % at 4096 query rows over 4096 keys).  Only for caches that fit a modest workspace.
+    pl.predeq_offset = (pl.part_o_bytes + pl.part_ml_bytes + 255) / 256 * 256;
+    pl.predeq_bytes = 0;
+    const size_t dq = (size_t)a->kv_rows * 512 * sizeof(uint16_t);
+    if (rows * a->topk >= 8 * a->kv_rows && dq <= SFA_PREDEQ_MAX_BYTES && pl.predeq_offset + dq <= max_bytes) pl.predeq_bytes = dq;
     return pl;
 }
+
+size_t sfa_ws_bytes(const SfaPlan &pl) { return pl.predeq_bytes ? pl.predeq_offset + pl.predeq_bytes : pl.part_o_bytes + pl.part_ml_bytes; }
 
 constexpr int PACKED_ROW_BYTES = 656;     // 512 int8 | 64 bf16 | 4 fp32
 
@@ -246,9 +260,18 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
             if (reinterpret_cast<uintptr_t>(ptr) & 3)
                 return fail(PTO_E_INVALID_ARG, "sfa: index, block-table and length pointers must be 4-byte aligned");
     }
-    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
+    const bool predeq = pl.predeq_bytes != 0 && !kn_bf16;
+    const size_t need = predeq ? sfa_ws_bytes(pl) : pl.part_o_bytes + pl.part_ml_bytes;
     if (need > 0 && (!a->workspace || a->workspace_bytes < need))
         return fail(PTO_E_WORKSPACE, "sfa: workspace of %zu bytes required, %zu given", need, a->workspace ? a->workspace_bytes : (size_t)0);
+    if (predeq) {
+        uint16_t *dq = reinterpret_cast<uint16_t *>(static_cast<char *>(a->workspace) + pl.predeq_offset);
+        hipError_t e = pto::sfa_dequant_cache(kn, kn_pitch, ksc, ksc_pitch, dq, a->kv_rows, static_cast<hipStream_t>(hip_stream));
+        if (e != hipSuccess) return fail(PTO_E_LAUNCH, "sfa: launch failed: %s", hipGetErrorString(e));
+        kn = reinterpret_cast<const int8_t *>(dq);
+        kn_pitch = 1024;
+        kn_bf16 = true;
+    }
 
     pto::SfaParams p;
     p.q_nope = static_cast<const uint16_t *>(a->query_nope);
@@ -265,7 +288,7 @@ int sfa_enqueue(const PtoSfaQuantArgs *a, const int8_t *kn, int kn_pitch, const 
     p.act = a->kv_act_seqs;
     p.out = static_cast<uint16_t *>(a->attention_out);
     p.part_o = static_cast<uint16_t *>(a->workspace);
-    p.part_ml = need > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
+    p.part_ml = pl.part_ml_bytes > 0 ? reinterpret_cast<float *>(static_cast<char *>(a->workspace) + pl.part_o_bytes) : nullptr;
     p.kv_rows = a->kv_rows;
     p.T = (int)(a->b * a->s1);
     p.S1 = (int)a->s1;
@@ -395,7 +418,7 @@ int pto_sfa_quant_workspace_bytes(const PtoSfaQuantArgs *a, size_t *bytes)
     int rc = sfa_check(a);
     if (rc != PTO_OK) return rc;
     const SfaPlan pl = sfa_plan(a);
-    *bytes = pl.part_o_bytes + pl.part_ml_bytes;
+    *bytes = sfa_ws_bytes(pl);
     return PTO_OK;
 }
 
@@ -418,7 +441,7 @@ int pto_sfa_quant_launch_static(const PtoSfaQuantArgs *a, void *hip_stream)
         !a->block_table || !a->kv_act_seqs || !a->attention_out)
         return fail(PTO_E_INVALID_ARG, "sfa: a tensor pointer is NULL");
     const SfaPlan pl = sfa_plan(a, SFA_STATIC_SCRATCH_BYTES);
-    const size_t need = pl.part_o_bytes + pl.part_ml_bytes;
+    const size_t need = sfa_ws_bytes(pl);
     if (need > SFA_STATIC_SCRATCH_BYTES)
         return fail(PTO_E_WORKSPACE,
                     "sfa: the key splits of this shape need %zu bytes of scratch, the built-in array holds %zu; use "

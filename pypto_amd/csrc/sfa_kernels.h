@@ -35,5 +35,8 @@ struct SfaParams {
 };
 
 hipError_t sfa_launch(const SfaParams &p, hipStream_t stream);
+// the int8 latent part of `rows` cache rows as bf16 [rows, 512] (what the attention kernel de-quantises them to)
+hipError_t sfa_dequant_cache(const int8_t *kn, int kn_pitch, const uint8_t *ksc, int ksc_pitch, uint16_t *out, long long rows,
+                             hipStream_t stream);
 
 }  // namespace pto

@@ -940,6 +940,24 @@ __global__ __launch_bounds__(256) void sfa_combine_many_kernel(const SfaParams p
     *reinterpret_cast<u32x4 *>(p.out + ((size_t)t * p.NQ + head) * DN + 8 * c8) = outv;
 }
 
+// De-quantises whole cache rows once: out[row][c] = bf16_rne(float(int8) * scale[c / 128]), the values the attention
+// kernel forms on the way into LDS.  One wave per row, a lane per eight channels.  For launches that select every
+// key many times over (a prefill chunk attends its few thousand keys from thousands of query rows), after which
+// the kernel takes its bf16-cache form on these rows: the same bits, without the per-tile conversion.
+__global__ __launch_bounds__(256) void sfa_dequant_cache_kernel(const int8_t *kn, const int kn_pitch, const uint8_t *ksc, const int ksc_pitch,
+                                                                uint16_t *out, const long long rows)
+{
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int l = threadIdx.x & 63;
+    const u32x2 raw = *reinterpret_cast<const u32x2 *>(kn + (size_t)row * kn_pitch + 8 * l);
+    const float sc = reinterpret_cast<const float *>(ksc + (size_t)row * ksc_pitch)[l >> 4];
+    const float bias = -128.0f * sc;
+    const u32x2 lo = dequant4(raw[0], sc, bias), hi = dequant4(raw[1], sc, bias);
+    const u32x4 v = {lo[0], lo[1], hi[0], hi[1]};
+    *reinterpret_cast<u32x4 *>(out + (size_t)row * DN + 8 * l) = v;
+}
+
 }  // namespace
 
 hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
@@ -976,6 +994,13 @@ hipError_t sfa_launch(const SfaParams &p, hipStream_t stream)
         e = hipGetLastError();
     }
     return e;
+}
+
+hipError_t sfa_dequant_cache(const int8_t *kn, int kn_pitch, const uint8_t *ksc, int ksc_pitch, uint16_t *out, long long rows,
+                             hipStream_t stream)
+{
+    hipLaunchKernelGGL(sfa_dequant_cache_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, kn, kn_pitch, ksc, ksc_pitch, out, rows);
+    return hipGetLastError();
 }
 
 }  // namespace pto
