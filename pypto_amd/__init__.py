@@ -25,4 +25,4 @@ from .sparse_attention_antiquant_impl import sparse_attention_antiquant_d, spars
 from .sparse_flash_attention_quant_impl import (SaTileShapeConfig, sparse_flash_attention_quant_d,  # noqa: F401
                                                 sparse_flash_attention_quant_p)
 
-__version__ = "0.5.1"
+__version__ = "0.6.0"

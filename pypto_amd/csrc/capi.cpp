@@ -408,7 +408,7 @@ extern "C" {
 
 const char *pto_last_error(void) { return g_err; }
 
-const char *pto_version(void) { return "0.5.1"; }
+const char *pto_version(void) { return "0.6.0"; }
 
 int pto_abi_revision(void) { return PTO_ABI_REVISION; }
 

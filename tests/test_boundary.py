@@ -53,7 +53,10 @@ def test_pybind_workspace_and_argument_errors():
     C = _native.load()
     # 32 rows x 8 splits x 128 heads x (512 fp16 + 2 fp32)
     assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 20, 0.04, 8) == 32 * 8 * 128 * (512 * 2 + 8)
-    assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 0      # no split needed
+    # more rows than compute units, a cache much larger than the selections: neither split nor de-quantised copy
+    assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 1 << 21, 0.04, 0) == 0
+    # prefill-shaped (every cache row selected by many query rows): one bf16 copy of the 4096 cache rows
+    assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 4096 * 512 * 2
     assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * (32768 + 2048) * 4
     # prolog: 4 int32 partial projections [t, 8192] + 112 block sums [t, 192] fp32
     assert C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 64, 1 << 20) == 4 * 8 * 8192 * 4 + 112 * 8 * 192 * 4
