@@ -53,15 +53,19 @@ namespace {
 static_assert(LIP_KSPLIT == QPROJ_KSPLIT, "workspace sizing and the projection job disagree");
 
 // ---------------------------------------------------------------------------------------------
-// Hidden-axis jobs: block c of 64 rows, tokens t0, t0+1.  Even jobs take wk (lane l: columns 2l,
+// Hidden-axis jobs: block c of 64 rows, tokens t0 .. t0+XTOK-1.  Even jobs take wk (lane l: columns 2l,
 // 2l+1), odd jobs w_proj (lane l: column l).  The block of weights (contiguous in memory) travels to
-// the wave's LDS region by LDS-DMA, the two token slices are converted to fp32 on the way in; the
-// product loop reads weights per lane and the hidden states as broadcasts.
+// the wave's LDS region by LDS-DMA, the token slices are converted to fp32 on the way in; the
+// product loop reads weights per lane and the hidden states as broadcasts.  XTOK = 2 gives a batch of up to
+// eight tokens one job per wave of the launch; larger batches take 4 or 8 tokens per staged block, so that the
+// launch stays one round of workgroups and a block is staged once per 4 or 8 tokens (the sums, one per token
+// and column over ascending rows, do not depend on XTOK).
 constexpr int XW_BYTES = LIP_XBLOCK * LIP_DIM * 2;     // 16 KiB: a block of wk
-constexpr int XTOK = 2;                               // tokens per hidden-axis job
-constexpr int X_REGION_BYTES = XW_BYTES + XTOK * LIP_XBLOCK * 4;
+constexpr int XTOK_MAX = 8;                           // most tokens per hidden-axis job
+constexpr int X_REGION_BYTES = XW_BYTES + XTOK_MAX * LIP_XBLOCK * 4;
 constexpr int LIN_XWAVES = 4;
 
+template <int XTOK>
 __device__ __forceinline__ void x_linear_job(const LipParams &p, uint8_t *region, const int job)
 {
     const int l = threadIdx.x & 63;
@@ -83,19 +87,22 @@ __device__ __forceinline__ void x_linear_job(const LipParams &p, uint8_t *region
         o = o < bytes - 16 ? o : bytes - 16;            // lanes past the end re-read its last 16 bytes
         dma16(wsrc + o, wdst + off);
     }
-    {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + l/32
-        const int t = t0 + (l >> 5);
+#pragma unroll
+    for (int tp = 0; tp < XTOK; tp += 2) {   // lane l: hidden states k0 + 2*(l%32), +1 of token t0 + tp + l/32
+        const int t = t0 + tp + (l >> 5);
         const int tt = t < p.T ? t : p.T - 1;
         const uint32_t xv = reinterpret_cast<const uint32_t *>(p.x + (size_t)tt * p.h + k0)[l & 31];
         f32x2 v = {__uint_as_float(xv << 16), __uint_as_float(xv & 0xffff0000u)};
-        *reinterpret_cast<f32x2 *>(xs + (l >> 5) * LIP_XBLOCK + 2 * (l & 31)) = v;
+        *reinterpret_cast<f32x2 *>(xs + (tp + (l >> 5)) * LIP_XBLOCK + 2 * (l & 31)) = v;
     }
     VM_WAIT(0);
     // the wave reads back only what it wrote or requested itself: no barrier
 
     if (!proj) {
         const uint32_t *wl = reinterpret_cast<const uint32_t *>(region) + l;
-        float a0[XTOK] = {0.f, 0.f}, a1[XTOK] = {0.f, 0.f};
+        float a0[XTOK], a1[XTOK];
+#pragma unroll
+        for (int t = 0; t < XTOK; ++t) a0[t] = a1[t] = 0.f;
 #pragma unroll 2
         for (int kk = 0; kk < LIP_XBLOCK; kk += 4) {
             f32x4 xv[XTOK];
@@ -122,7 +129,9 @@ __device__ __forceinline__ void x_linear_job(const LipParams &p, uint8_t *region
     } else {
         const bool pl = l < p.n_heads;
         const uint16_t *wl = reinterpret_cast<const uint16_t *>(region) + (pl ? l : 0);
-        float a2[XTOK] = {0.f, 0.f};
+        float a2[XTOK];
+#pragma unroll
+        for (int t = 0; t < XTOK; ++t) a2[t] = 0.f;
 #pragma unroll 2
         for (int kk = 0; kk < LIP_XBLOCK; kk += 4) {
             f32x4 xv[XTOK];
@@ -149,7 +158,7 @@ constexpr int lin_lds_bytes()
 
 // Workgroup of six waves, no dependencies among them except the final pairwise sum of the two query
 // waves: waves 0 and 1 run the two halves of query job blockIdx.x, waves 2..5 walk the hidden-axis jobs.
-template <int HS>
+template <int HS, int XTOK>
 __global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const LipParams p, const int q_jobs, const int x_jobs)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lip_smem[lin_lds_bytes<HS>()];
@@ -170,7 +179,7 @@ __global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const
         if (w == 1) q_pair_park(region, l, acc);
     } else if (w >= 2) {
         uint8_t *xregion = lip_smem + 2 * lin_region_bytes<HS>() + (w - 2) * X_REGION_BYTES;
-        for (int j = job * LIN_XWAVES + (w - 2); j < x_jobs; j += gridDim.x * LIN_XWAVES) x_linear_job(p, xregion, j);
+        for (int j = job * LIN_XWAVES + (w - 2); j < x_jobs; j += gridDim.x * LIN_XWAVES) x_linear_job<XTOK>(p, xregion, j);
     }
     __syncthreads();
     if (qwave && w == 0) q_pair_store<HS>(qp, lip_smem, job, l, acc);
@@ -285,18 +294,28 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
         hipLaunchKernelGGL(lip_xlinear_group_kernel, dim3((unsigned)(2 * ngroups * tgroups)), dim3(64 * XL_WAVES), 0, stream, p, ngroups);
         return hipGetLastError();
     }
-    const int x_jobs = 2 * (p.h / LIP_XBLOCK) * ((p.T + XTOK - 1) / XTOK);
+    // tokens per hidden-axis job: 2 up to eight tokens, 4 up to sixteen, 8 beyond (a workgroup holds a CU, so
+    // more jobs than one round of workgroups has waves run as further rounds)
+    const int xtok = p.T <= 8 ? 2 : (p.T <= 16 ? 4 : 8);
+    const int x_jobs = 2 * (p.h / LIP_XBLOCK) * ((p.T + xtok - 1) / xtok);
     // enough workgroups that each hidden-axis wave gets about one job, never fewer than the query jobs
     int wgs = (x_jobs + LIN_XWAVES - 1) / LIN_XWAVES;
     wgs = wgs > 4096 ? 4096 : wgs;
     wgs = wgs > q_jobs ? wgs : q_jobs;
     const dim3 grid1((unsigned)wgs), block1(128 + 64 * LIN_XWAVES);
+#define LIP_LINEAR(HS)                                                                                              \
+    switch (xtok) {                                                                                                \
+    case 2: hipLaunchKernelGGL((lip_linear_kernel<HS, 2>), grid1, block1, 0, stream, p, q_jobs, x_jobs); break;  \
+    case 4: hipLaunchKernelGGL((lip_linear_kernel<HS, 4>), grid1, block1, 0, stream, p, q_jobs, x_jobs); break;  \
+    default: hipLaunchKernelGGL((lip_linear_kernel<HS, 8>), grid1, block1, 0, stream, p, q_jobs, x_jobs); break; \
+    }
     switch (steps) {
-    case 4: hipLaunchKernelGGL(lip_linear_kernel<2>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
-    case 8: hipLaunchKernelGGL(lip_linear_kernel<4>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
-    case 12: hipLaunchKernelGGL(lip_linear_kernel<6>, grid1, block1, 0, stream, p, q_jobs, x_jobs); break;
+    case 4: LIP_LINEAR(2) break;
+    case 8: LIP_LINEAR(4) break;
+    case 12: LIP_LINEAR(6) break;
     default: return hipErrorInvalidValue;
     }
+#undef LIP_LINEAR
     return hipGetLastError();
 }
 

@@ -61,6 +61,8 @@ def assert_exact(got, ref, what):
     (1, 1, [77], dict(h=128, q_lora_rank=1024, n_heads=3)),               # one token, odd head count
     (3, 1, [5, 128, 129], dict(h=512, q_lora_rank=1536, n_heads=8, affine_ln=True)),   # gamma/beta drawn at random
     (5, 7, [900] * 5, dict(h=192, q_lora_rank=512, n_heads=2)),           # 35 tokens: two token blocks, ragged groups of 4
+    (3, 5, [700] * 3, dict(h=192, q_lora_rank=512, n_heads=2)),           # 15 tokens: four tokens per hidden-axis job, the last job ragged
+    (32, 1, [300] * 32, dict(h=256, q_lora_rank=512, n_heads=4)),         # 32 tokens: eight tokens per hidden-axis job
 ])
 def test_prolog_small_shapes_bit_exact(b, s1, act, kw):
     inp = gen_indexer_prolog_inputs(b, s1, act, seed=3 * b + s1, **kw)
