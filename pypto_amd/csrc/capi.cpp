@@ -145,7 +145,15 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a, const size_t max_bytes = ~(size_t)0)
         const long long xcd_rows = (rows + 7) / 8;
         const int max_split = tiles / 4 > 0 ? tiles / 4 : 1;
         double best = -1.0;
-        for (int s = 1; s <= max_split; ++s) {
+        if (cus % 8 != 0) {
+            // not the layout the schedule model describes (a partitioned device, another part): one workgroup per
+            // compute unit, as many splits as that takes
+            const long long per_split = rows * pl.hgroups;
+            ns = (int)((cus + per_split - 1) / per_split);
+            ns = ns > max_split ? max_split : ns;
+            while (ns > 1 && ns > min_split && (size_t)rows * ns * a->nq * (512 * sizeof(uint16_t) + 2 * sizeof(float)) > max_bytes) --ns;
+        }
+        for (int s = 1; s <= max_split && cus % 8 == 0; ++s) {
             if (s > 1 && s >= min_split && (size_t)rows * s * a->nq * (512 * sizeof(uint16_t) + 2 * sizeof(float)) > max_bytes) break;
             const long long rounds = (xcd_rows * pl.hgroups * s + xcd_cus - 1) / xcd_cus;
             const double merge = s == 1 ? 0.0 : 1.0 + 0.01 * (double)rows * s * pl.hgroups;
@@ -169,7 +177,7 @@ SfaPlan sfa_plan(const PtoSfaQuantArgs *a, const size_t max_bytes = ~(size_t)0)
         const int cus = cu_count() > 0 ? cu_count() : 256;
         const long long xcd_cus = cus / 8 > 0 ? cus / 8 : 1;
         const long long xcd_rows = (rows + 7) / 8;
-        const long long per_round = xcd_cus / pl.hgroups;                 // rows of an XCD that one round holds
+        const long long per_round = cus % 8 == 0 ? xcd_cus / pl.hgroups : 0;   // rows of an XCD that one round holds
         const long long full = per_round > 0 ? xcd_rows / per_round : 0;
         const long long rem = per_round > 0 ? xcd_rows - full * per_round : 0;
         if (full >= 1 && rem >= 1) {

@@ -185,10 +185,11 @@ __global__ __launch_bounds__(128 + 64 * LIN_XWAVES) void lip_linear_kernel(const
     if (qwave && w == 0) q_pair_store<HS>(qp, lip_smem, job, l, acc);
 }
 
+template <int TB>
 __global__ __launch_bounds__(256) void lip_qproj_prefill_kernel(const QProj p, const int njobs)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lds[QPF_LDS];
-    q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+    q_prefill_body<TB>(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
 // The fixed-order sums over the hidden axis at prefill sizes (xlinear_fixed.h, the form that broadcasts the hidden
@@ -277,7 +278,9 @@ hipError_t lip_launch_linear(const LipParams &p, hipStream_t stream)
             hipLaunchKernelGGL(lip_qproj_prefill256_kernel, dim3((unsigned)njobs256), dim3(512), 0, stream, qp, njobs256);
         } else {
             const int njobs = q_prefill_jobs(qp);
-            hipLaunchKernelGGL(lip_qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+            const dim3 g((unsigned)njobs), b(256);
+            if (q_prefill_token_blocks(p.T) == 2) hipLaunchKernelGGL(lip_qproj_prefill_kernel<2>, g, b, 0, stream, qp, njobs);
+            else hipLaunchKernelGGL(lip_qproj_prefill_kernel<4>, g, b, 0, stream, qp, njobs);
         }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;

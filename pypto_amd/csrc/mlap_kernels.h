@@ -20,7 +20,10 @@ constexpr int MLAP_MFMA_MIN_TOKENS = 9;    // from here on the stages take their
                                            // per head (the decode forms work on 8 tokens at a time and their cost grows with every
                                            // 8 tokens; those forms cost the same from 9 to 128 tokens, about what 8 tokens cost here)
 constexpr int MLAP_UNSPLIT_MIN_TOKENS = 64;   // with absorb_exact the projection still runs unsplit from here on
-constexpr int MLAP_XM_MAX_SPLITS = 8;      // ranges of the hidden axis (partial sums per token) of that form, at most
+// ranges of the hidden axis (partial sums per token) of that form, at most.  With a single token tile the sixteen
+// matrix-core slabs x 14 ranges and the rope columns' 32 workgroups are one workgroup per compute unit of an
+// MI355X, every one requesting weights from the start (8 ranges: 32 tokens 44.6 us per pass, 14: 40.9, 20 or 28: 43.3)
+constexpr int MLAP_XM_MAX_SPLITS = 14;
 
 // rows [T, q_lora + 576] of partial sums over the hidden axis the workspace holds: the group sums of the
 // fixed-order form, or the ranges of the matrix-core form where that may run

@@ -318,10 +318,12 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj pa, const int nj
     }
 }
 
+// TB: token blocks per tile (prolog_common.h)
+template <int TB>
 __global__ __launch_bounds__(256) void qproj_prefill_kernel(const QProj p, const int njobs)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lds[QPF_LDS];
-    q_prefill_body(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
+    q_prefill_body<TB>(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
 __global__ __launch_bounds__(512) void qproj_prefill256_kernel(const QProj p, const int njobs)
@@ -374,8 +376,8 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
     if (rider != nullptr && !mlap_takes_rider(p)) return hipErrorInvalidValue;
     const MlapRider rd = rider != nullptr ? *rider : MlapRider{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (mlap_prefill_forms(p)) {
-        // prefill sizes: the sums over the hidden axis on the matrix cores, up to four partial sums per token
-        // as many ranges as give about two workgroups per compute unit (one is resident at a time, by its LDS)
+        // prefill sizes: the sums over the hidden axis on the matrix cores, in as many ranges of the hidden axis
+        // (partial sums per token) as give about two workgroups per compute unit, MLAP_XM_MAX_SPLITS at most
         const int nchunks = p.h / XM_KC;
         const int ttiles = (p.T + XM_TOK - 1) / XM_TOK;
         const int cus = cu_count();
@@ -412,7 +414,12 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
             return hipGetLastError();
         }
         const int njobs = q_prefill_jobs(qp);
-        hipLaunchKernelGGL(qproj_prefill_kernel, dim3((unsigned)njobs), dim3(256), 0, stream, qp, njobs);
+        const dim3 g((unsigned)njobs), b(256);
+        switch (q_prefill_token_blocks(p.T)) {
+        case 1: hipLaunchKernelGGL(qproj_prefill_kernel<1>, g, b, 0, stream, qp, njobs); break;
+        case 2: hipLaunchKernelGGL(qproj_prefill_kernel<2>, g, b, 0, stream, qp, njobs); break;
+        default: hipLaunchKernelGGL(qproj_prefill_kernel<4>, g, b, 0, stream, qp, njobs);
+        }
         return hipGetLastError();
     }
     const int qjobs_a = qp.nslabs * QPROJ_KSPLIT * ((p.T + 31) / 32);

@@ -60,6 +60,18 @@ __device__ __forceinline__ float bf16_round_f32(const float v)
 // the eight rows of a half-wave's read fall on different banks; the LDS-DMA requests place the pieces that way.
 __device__ __forceinline__ int q_tr_piece_swizzle(const int row) { return 2 * ((row >> 1) & 3); }
 
+// the operand of product i alone
+__device__ __forceinline__ i32x4 q_build_a_tr_one(const uint8_t *tile, const int s, const int l, const int i)
+{
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    const int x = (l >> 2) & 3;
+    const uint8_t *pi = tile + (32 * s + 16 * (l >> 5) + ((l & 15) >> 1)) * 128 + 16 * ((l >> 4) & 1) + 8 * (l & 1) + 32 * (i ^ x);
+    const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)pi);
+    const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(lds_byte_t *)(pi + 8 * 128));
+    const i32x4 a = {lo[0], lo[1], hi[0], hi[1]};
+    return a;
+}
+
 __device__ __forceinline__ void q_build_a_tr(const uint8_t *tile, const int s, const int l, i32x4 (&a)[4])
 {
     typedef int v2i __attribute__((ext_vector_type(2)));
@@ -204,19 +216,20 @@ __device__ __forceinline__ void q_pair_park(uint8_t *region, const int l, const 
 // of this lane's token (q_build_a_tr).  tbase: first of the wave's 32 tokens; col0: first of its 128 columns.
 constexpr int Q_STAGE_PITCH = 272;                     // bytes between token rows: 16-byte aligned, 4 banks apart
 constexpr int Q_STAGE_BYTES = 32 * Q_STAGE_PITCH;
-__device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16 (&acc)[4], const int tbase, const int col0, const int l,
-                                                    uint8_t *stage)
+// products i0 .. i0+NP-1 of a wave (columns 32*i0 .. of the 128 at col0) go to the staging area of their token block
+template <int NP>
+__device__ __forceinline__ void q_stage_products(const QProj &p, const i32x16 (&acc)[NP], const int i0, const int tbase, const int col0, const int l,
+                                                 uint8_t *stage)
 {
-    const int ncols = p.nslabs * 128;
     const int t = tbase + (l & 31);
     const float ts = p.tok_scale[t < p.T ? t : p.T - 1];
     const float *cs = p.col_scale + col0;
     uint8_t *mine = stage + (l & 31) * Q_STAGE_PITCH;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NP; ++i)
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
-            const int col = 32 * i + 8 * rg + 4 * (l >> 5);
+            const int col = 32 * (i0 + i) + 8 * rg + 4 * (l >> 5);
             const f32x4 c = *reinterpret_cast<const f32x4 *>(cs + col);
             float v[4];
 #pragma unroll
@@ -224,14 +237,26 @@ __device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16
             const u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
             *reinterpret_cast<u32x2 *>(mine + 2 * col) = o;
         }
-    // the wave reads back what it wrote itself: LDS operations of a wave stay in order
+}
+// rows 4*k .. 4*k+3 (k = k_begin .. k_end-1) of a staged token block leave as whole 256-byte rows
+__device__ __forceinline__ void q_store_rows(const QProj &p, const int tbase, const int col0, const int l, const uint8_t *stage, const int k_begin,
+                                             const int k_end)
+{
+    const int ncols = p.nslabs * 128;
     uint16_t *dst = reinterpret_cast<uint16_t *>(p.part) + col0 + 8 * (l & 15);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = k_begin; k < k_end; ++k) {
         const int row = 4 * k + (l >> 4);
         const u32x4 v = *reinterpret_cast<const u32x4 *>(stage + row * Q_STAGE_PITCH + 16 * (l & 15));
         if (tbase + row < p.T) *reinterpret_cast<u32x4 *>(dst + (size_t)(tbase + row) * ncols) = v;
     }
+}
+__device__ __forceinline__ void q_store_dequantised(const QProj &p, const i32x16 (&acc)[4], const int tbase, const int col0, const int l,
+                                                    uint8_t *stage)
+{
+    q_stage_products<4>(p, acc, 0, tbase, col0, l, stage);
+    // the wave reads back what it wrote itself: LDS operations of a wave stay in order
+    q_store_rows(p, tbase, col0, l, stage, 0, 8);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -248,65 +273,92 @@ constexpr int QPF_BUF = QPF_TILE + 4 * QPF_TOK;
 constexpr int QPF_LDS = 2 * QPF_BUF;                   // 64 KiB
 
 __host__ __device__ inline int q_prefill_jobs(const QProj &p) { return p.nslabs * ((p.T + 127) / 128); }
+// token blocks per tile of the form to take: a launch of one tile of one or two blocks has forms of its own
+__host__ __device__ inline int q_prefill_token_blocks(const int T) { return T <= 32 ? 1 : (T <= 64 ? 2 : 4); }
 
-// job: the blocks of a slab are neighbours in the job order
+// job: the blocks of a slab are neighbours in the job order.
+// TB: blocks of 32 tokens the tile holds.  TB = 4 is the form described above.  A launch of at most 32 or 64 tokens
+// (one tile of TB = 1 or 2 blocks per slab) shares a token block among 4 / TB waves, each with TB of the four
+// 32-column products: a wave then issues 4 or 8 products per chunk instead of 16 on padding tokens, and the
+// kernel's time is its requests' and no longer a wave's products'.  Same integer sums, same conversion.
+template <int TB = 4>
 __device__ __forceinline__ void q_prefill_body(const QProj &p, const int job, uint8_t *lds)
 {
+    static_assert(TB == 1 || TB == 2 || TB == 4, "token blocks per tile");
+    constexpr int WPB = 4 / TB;                        // waves that share a token block
     const int l = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tb = w % TB;                             // this wave's token block
+    const int i0 = (w / TB) * TB;                      // its first product (32 columns each)
     const int ncols = p.nslabs * 128;
-    const int ttiles = (p.T + 127) / 128;
+    const int ttiles = (p.T + 32 * TB - 1) / (32 * TB);
     const int slab = job / ttiles;
-    const int t = (job % ttiles) * 128 + 32 * w + (l & 31);
+    const int tile0 = (job % ttiles) * (32 * TB);
     const int nch = p.q_lora / (32 * QPF_STEPS);
     // token operands: a request brings 128 bytes (the chunk's four steps) of 8 tokens -- whole lines; as 32 tokens x 32
     // bytes a request runs at half the rate.  Lane l fills piece l % 8 of token row l / 8 with piece (l % 8) ^ (l / 8)
-    // of that token, so that the operand reads of 8 consecutive tokens fall on different banks.
-    const int8_t *tsrc[4];
+    // of that token, so that the operand reads of 8 consecutive tokens fall on different banks.  The four requests
+    // of a token block are dealt to the waves that share it.
+    const int8_t *tsrc[TB];
+    int treq[TB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int tq = (job % ttiles) * 128 + 32 * w + 8 * i + (l >> 3);
+    for (int k = 0; k < TB; ++k) {
+        const int i = (w / TB) + WPB * k;              // request (eight tokens) of block tb
+        treq[k] = i;
+        int tq = tile0 + 32 * tb + 8 * i + (l >> 3);
         tq = tq < p.T ? tq : p.T - 1;                  // rows past the end repeat the last token and are not stored
-        tsrc[i] = p.q_norm + (size_t)tq * p.q_lora + 16 * ((l & 7) ^ (l >> 3));
+        tsrc[k] = p.q_norm + (size_t)tq * p.q_lora + 16 * ((l & 7) ^ (l >> 3));
     }
     // lane l of a tile request fills piece l % 8 of row l / 8 of its eight rows: with the piece that belongs there (q_build_a_tr)
     const int8_t *wsrc = p.w + (size_t)(32 * w + (l >> 3)) * ncols + slab * 128 + 16 * ((l & 7) ^ q_tr_piece_swizzle(l >> 3));
     const uint32_t base = (uint32_t)(uintptr_t)(lds_byte_t *)lds;
-    auto issue = [&](const int c) {
-        const uint32_t buf = base + (c & 1) * QPF_BUF;
+    auto issue = [&](const int c, const int b) {
+        const uint32_t buf = base + b * QPF_BUF;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(tsrc[i] + c * (32 * QPF_STEPS), buf + QPF_TILE + w * QPF_TOK + 1024 * i);
+        for (int k = 0; k < TB; ++k) dma16(tsrc[k] + c * (32 * QPF_STEPS), buf + QPF_TILE + tb * QPF_TOK + 1024 * treq[k]);
 #pragma unroll
         for (int i = 0; i < 4; ++i) dma16(wsrc + ((size_t)c * (32 * QPF_STEPS) + 8 * i) * ncols, buf + 1024 * (4 * w + i));
     };
-    i32x16 acc[4];
+    i32x16 acc[TB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TB; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][r] = 0;
-    issue(0);
+    auto products = [&](const uint8_t *buf) {
+#pragma unroll
+        for (int s = 0; s < QPF_STEPS; ++s) {
+            const i32x4 b = *reinterpret_cast<const i32x4 *>(buf + QPF_TILE + tb * QPF_TOK + (l & 31) * 128 + 16 * ((2 * s + (l >> 5)) ^ (l & 7)));
+            if (TB == 4) {
+                i32x4 a[4];
+                q_build_a_tr(buf, s, l, a);
+#pragma unroll
+                for (int i = 0; i < TB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TB; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q_build_a_tr_one(buf, s, l, i0 + i), b, acc[i], 0, 0, 0);
+            }
+        }
+    };
+    constexpr int PER_CHUNK = TB + 4;                  // a wave's requests of a chunk
+    issue(0, 0);
 #pragma unroll 1
     for (int c = 0; c < nch; ++c) {
         if (c + 1 < nch) {
-            issue(c + 1);
-            VM_WAIT(QPF_STEPS + 4);
+            issue(c + 1, (c + 1) & 1);
+            VM_WAIT(PER_CHUNK);
         } else {
             VM_WAIT(0);
         }
         __syncthreads();                               // every wave's share of chunk c has landed
-        const uint8_t *buf = lds + (c & 1) * QPF_BUF;
-#pragma unroll
-        for (int s = 0; s < QPF_STEPS; ++s) {
-            i32x4 a[4];
-            q_build_a_tr(buf, s, l, a);
-            const i32x4 b = *reinterpret_cast<const i32x4 *>(buf + QPF_TILE + w * QPF_TOK + (l & 31) * 128 + 16 * ((2 * s + (l >> 5)) ^ (l & 7)));
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b, acc[i], 0, 0, 0);
-        }
+        products(lds + (c & 1) * QPF_BUF);
         __syncthreads();                               // chunk c + 2 goes where chunk c was read
     }
     static_assert(4 * Q_STAGE_BYTES <= QPF_LDS, "the staging areas reuse the chunk buffers");
-    q_store_dequantised(p, acc, t - (l & 31), slab * 128, l, lds + w * Q_STAGE_BYTES);   // past the loop's last barrier
+    // past the loop's last barrier: every token block has a staging area, filled by the waves that share the block
+    uint8_t *stage = lds + tb * Q_STAGE_BYTES;
+    q_stage_products<TB>(p, acc, i0, tile0 + 32 * tb, slab * 128, l, stage);
+    if (TB < 4) __syncthreads();                       // (a wave of the TB = 4 form reads back only what it wrote itself)
+    q_store_rows(p, tile0 + 32 * tb, slab * 128, l, stage, (w / TB) * 2 * TB, (w / TB + 1) * 2 * TB);
 }
 // The same projection for grids that fill the chip with larger tiles: a workgroup of eight waves per (256 columns,
 // 256 tokens); wave (wc, wt) holds columns 128*wc .. +127 x tokens 64*wt .. +63 (eight accumulators), so a weight

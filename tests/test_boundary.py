@@ -68,7 +68,7 @@ def test_pybind_workspace_and_argument_errors():
         C.li_prolog_quant_workspace_bytes(8, 7168, 1536, 65, 1 << 20)                # more than 64 heads
     # MLA prolog: 14 group sums [t, 1536 + 576] fp32 + 4 int32 partial projections [t, 128 * 192]
     assert C.mla_prolog_quant_workspace_bytes(8, 7168, 1536, 128, 1 << 16) == 14 * 8 * 2112 * 4 + 4 * 8 * 24576 * 4
-    # from 9 tokens on the partial sums over the hidden axis may be the matrix-core form's ranges (up to eight, one
+    # from 9 tokens on the partial sums over the hidden axis may be the matrix-core form's ranges (up to fourteen, one
     # per block of 64 hidden rows at most): a 192-wide hidden axis is one group but three ranges
     assert C.mla_prolog_quant_workspace_bytes(150, 192, 512, 2, 1 << 16) == 3 * 150 * 1088 * 4 + 4 * 150 * 384 * 4
     assert C.mla_prolog_quant_workspace_bytes(32, 192, 512, 2, 1 << 16) == 3 * 32 * 1088 * 4 + 4 * 32 * 384 * 4
