@@ -145,13 +145,14 @@ def test_config4_prefill_4096_tokens(c_oracle):
     assert_close_to_fp64_truth(out, gold, inp, [(0, 1), (0, 99), (0, 2046), (0, 2047), (0, 3333), (0, 4095)], "cfg4")
 
 
-@pytest.mark.parametrize("b,s1", [(300, 1), (128, 4)])
-def test_more_query_rows_than_compute_units(c_oracle, b, s1):
+@pytest.mark.parametrize("b,s1,n_q", [(300, 1, 128), (128, 4, 128), (300, 1, 160)])
+def test_more_query_rows_than_compute_units(c_oracle, b, s1, n_q):
     """Decode batches past one workgroup per compute unit (the operator's documented range reaches b = 128 with
-    s1 = 4, examples/models/deepseek_v32_exp/README.md:6-24): 300 rows, which the library splits so that the last
-    round of workgroups is not nearly empty, and 512 rows; every row against the golden."""
+    s1 = 4, examples/models/deepseek_v32_exp/README.md:6-24): 300 rows, which the library runs as full rounds of
+    whole rows plus the rows left over in pieces, and 512 rows; every row against the golden.  160 heads make two
+    head groups per row (the second partly filled), so that whole rows and pieces each take two workgroups."""
     act = [2048 + 37 * (i % 11) for i in range(b)]
-    inp = gen_sfa_inputs(b, s1, 128, act, topk=2048, seed=b + s1)
+    inp = gen_sfa_inputs(b, s1, n_q, act, topk=2048, seed=b + s1)
     out = run_sfa(inp)
     gold = golden(c_oracle, inp)
     check(out, gold, f"b={b} s1={s1}")
