@@ -55,6 +55,13 @@ def test_pybind_workspace_and_argument_errors():
     assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 20, 0.04, 8) == 32 * 8 * 128 * (512 * 2 + 8)
     # more rows than compute units, a cache much larger than the selections: neither split nor de-quantised copy
     assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 1 << 21, 0.04, 0) == 0
+    # the automatic split (a host without a device plans for 256 compute units in 8 XCDs): 32 rows in 8 pieces each;
+    # 200 rows whole; 300 rows as 256 whole rows and the other 44 in 5 pieces each; 260 rows as 256 whole rows and
+    # the other 4 in 16 pieces (a piece keeps at least four tiles of 32 keys)
+    assert C.sfa_quant_workspace_bytes(32, 1, 128, 1, 2048, 128, 512, 1 << 21, 0.04, 0) == 32 * 8 * 128 * (512 * 2 + 8)
+    assert C.sfa_quant_workspace_bytes(200, 1, 128, 1, 2048, 128, 32, 1 << 21, 0.04, 0) == 0
+    assert C.sfa_quant_workspace_bytes(300, 1, 128, 1, 2048, 128, 32, 1 << 21, 0.04, 0) == 44 * 5 * 128 * (512 * 2 + 8)
+    assert C.sfa_quant_workspace_bytes(260, 1, 128, 1, 2048, 128, 32, 1 << 21, 0.04, 0) == 4 * 16 * 128 * (512 * 2 + 8)
     # prefill-shaped (every cache row selected by many query rows): one bf16 copy of the 4096 cache rows
     assert C.sfa_quant_workspace_bytes(4096, 1, 128, 1, 2048, 128, 32, 4096, 0.04, 0) == 4096 * 512 * 2
     assert C.li_decode_workspace_bytes(4, 4, 64, 128, 1024, 128, 256, 2048, 0, 0, 0) == 4 * (32768 + 2048) * 4
