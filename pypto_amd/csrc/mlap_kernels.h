@@ -90,7 +90,12 @@ inline bool mlap_takes_rider(const MlapParams &p) { return !mlap_prefill_forms(p
 
 hipError_t mlap_launch(const MlapParams &p, hipStream_t stream);
 // all launches but the last, and the number of workgroups of the last (for the fused operator's last launch)
-hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider = nullptr);
+// lip_rider (prefill forms below 64 tokens only): the indexer prolog whose first launch's jobs -- fixed-order sums
+// over the hidden axis, split int8 projection -- ride in this operator's first and third launch
+struct LipParams;
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider = nullptr, const LipParams *lip_rider = nullptr);
+// whether the launches of `p` take such a rider
+inline bool mlap_takes_lip_rider(const MlapParams &p) { return mlap_prefill_forms(p) && p.T < 64; }
 int mlap_finish_wgs(const MlapParams &p);
 // the last launch alone; at prefill sizes (mlap_finish_is_prefill) it has a form of its own that the fused operator
 // launches beside, not inside, its own last launch

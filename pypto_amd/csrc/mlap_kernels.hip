@@ -37,9 +37,12 @@
 //                        128 x 128 or 256 x 256 tile over the whole reduction axis; results leave de-quantised.
 //   mlap_finish_prefill_kernel   per (head, run of 32-token blocks): the head's whole w_uk staged once
 //                        (prolog_finish.h), absorb product on the matrix cores.
+#include <cstring>
+
 #include "mlap_kernels.h"
 #include "prolog_common.h"
 #include "prolog_finish.h"
+#include "lip_xjob.h"
 #include "xlinear_fixed.h"
 #include "xlinear_mfma.h"
 
@@ -100,11 +103,27 @@ static_assert(XM_KC == MLAP_XBLOCK, "the workspace is sized in chunks of the hid
 // form; workgroup = (group of eight blocks, 16 tokens)): the reference's acceptance rule allows the rotated key no
 // outlier at all (deepseekv32_mla_prolog_quant.py:688: atol 1e-4, rtol 2^-7 per element, ratio 0), and a sum that
 // lands next to a bf16 rounding boundary in another order moves a small rotated value by more than that.
+// The fused prolog's rider: workgroups past the launch's own run the indexer prolog's fixed-order sums over the
+// hidden axis (lip_xjob.h), a wave per job, beside the matrix-core workgroups (two workgroups fit a compute unit).
+struct MlapXRider {
+    LipParams lip;
+    int wgs;        // rider workgroups (0: none)
+    int x_jobs;
+    int xtok;
+};
+constexpr int XM_RIDER_LDS = 4 * X_REGION_BYTES;
+constexpr int XM_KERNEL_LDS = XM_LDS > XM_RIDER_LDS ? XM_LDS : XM_RIDER_LDS;
 static_assert(XR_LDS <= XM_LDS, "the rope jobs fit the launch's LDS");
+static_assert(2 * XM_KERNEL_LDS <= 160 * 1024, "two workgroups share a compute unit");
 __global__ __launch_bounds__(256) void mlap_xlinear_mfma_kernel(const MlapParams p, const int nslabs, const int nsplit, const int rope_wgs,
-                                                                const int rope_groups)
+                                                                const int rope_groups, const int own_wgs, const MlapXRider rider)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t smem[XM_LDS];
+    __shared__ __attribute__((aligned(16))) uint8_t smem[XM_KERNEL_LDS];
+    if ((int)blockIdx.x >= own_wgs) {
+        const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        x_linear_jobs(rider.lip, smem + w * X_REGION_BYTES, ((int)blockIdx.x - own_wgs) * 4 + w, rider.wgs * 4, rider.x_jobs, rider.xtok);
+        return;
+    }
     if ((int)blockIdx.x < rope_wgs) {
         const int j = blockIdx.x;
         const int g = j % rope_groups;
@@ -318,11 +337,35 @@ __global__ __launch_bounds__(128) void qproj_kernel(const QProj pa, const int nj
     }
 }
 
-// TB: token blocks per tile (prolog_common.h)
-template <int TB>
-__global__ __launch_bounds__(256) void qproj_prefill_kernel(const QProj p, const int njobs)
+// TB: token blocks per tile (prolog_common.h).  HS > 0: workgroups past the launch's own run the fused prolog's
+// rider, the indexer prolog's split int8 projection (one job of a wave pair each, HS steps of 32 rows per half; the
+// other two waves only keep the barrier company), beside the tiles' workgroups (two workgroups fit a compute unit).
+template <int TB, int HS>
+__global__ __launch_bounds__(256) void qproj_prefill_kernel(const QProj p, const int njobs, const QProj rider)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[QPF_LDS];
+    constexpr int RIDER_LDS = HS > 0 ? 2 * lin_region_bytes<(HS > 0 ? HS : 1)>() : 0;
+    constexpr int LDS = QPF_LDS > RIDER_LDS ? QPF_LDS : RIDER_LDS;
+    static_assert(2 * LDS <= 160 * 1024, "two workgroups share a compute unit");
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS];
+    if (HS > 0 && (int)blockIdx.x >= njobs) {
+        constexpr int H = HS > 0 ? HS : 1;
+        const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        const int l = threadIdx.x & 63;
+        const int job = (int)blockIdx.x - njobs;
+        i32x16 acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+        uint8_t *region = lds + (w & 1) * lin_region_bytes<H>();
+        if (w < 2) {
+            q_half_job<H>(rider, region, job, w, acc);
+            if (w == 1) q_pair_park(region, l, acc);
+        }
+        __syncthreads();
+        if (w == 0) q_pair_store<H>(rider, lds, job, l, acc);
+        return;
+    }
     q_prefill_body<TB>(p, q_prefill_job_of((int)blockIdx.x, njobs), lds);
 }
 
@@ -367,13 +410,14 @@ hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream)
 
 int mlap_finish_wgs(const MlapParams &p) { return p.n_heads * 2 * ((p.T + MLAP_XTOK - 1) / MLAP_XTOK); }
 
-hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider)
+hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const MlapRider *rider, const LipParams *lip_rider)
 {
     const int nblk = p.h / MLAP_XBLOCK;
     int ngroups = (nblk + MLAP_XGROUP - 1) / MLAP_XGROUP;
     const int ngroups_fixed = ngroups;
     const int nslabs = p.q_lora / 128 + 5;
     if (rider != nullptr && !mlap_takes_rider(p)) return hipErrorInvalidValue;
+    if (lip_rider != nullptr && !mlap_takes_lip_rider(p)) return hipErrorInvalidValue;
     const MlapRider rd = rider != nullptr ? *rider : MlapRider{nullptr, nullptr, nullptr, nullptr, nullptr, 0};
     if (mlap_prefill_forms(p)) {
         // prefill sizes: the sums over the hidden axis on the matrix cores, in as many ranges of the hidden axis
@@ -391,8 +435,20 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
         const int per_slab = ngroups * ttiles;
         const int wgs = 8 * ((mslabs >> 3) * per_slab + ((mslabs & 7) * per_slab + 7) / 8);   // the kernel's XCD-wise job order
         const int rope_wgs = (ngroups_fixed * ((p.T + XD_TOK - 1) / XD_TOK) + 7) / 8 * 8;
-        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)(rope_wgs + wgs)), dim3(256), 0, stream, p, mslabs, ngroups, rope_wgs,
-                           ngroups_fixed);
+        MlapXRider xr;
+        xr.wgs = 0;
+        xr.x_jobs = xr.xtok = 0;
+        if (lip_rider != nullptr) {
+            xr.lip = *lip_rider;
+            xr.xtok = lip_xtok(lip_rider->T);
+            xr.x_jobs = lip_x_jobs(*lip_rider, xr.xtok);
+            xr.wgs = (xr.x_jobs + 3) / 4;
+            xr.wgs = xr.wgs > 2 * cus ? 2 * cus : xr.wgs;
+        } else {
+            std::memset(&xr.lip, 0, sizeof xr.lip);
+        }
+        hipLaunchKernelGGL(mlap_xlinear_mfma_kernel, dim3((unsigned)(rope_wgs + wgs + xr.wgs)), dim3(256), 0, stream, p, mslabs, ngroups, rope_wgs,
+                           ngroups_fixed, rope_wgs + wgs, xr);
     } else {
         const int tgroups = (p.T + MLAP_XTOK - 1) / MLAP_XTOK;
         const int xslabs = nslabs + (rider != nullptr ? 1 : 0);
@@ -415,10 +471,29 @@ hipError_t mlap_launch_front(const MlapParams &p, hipStream_t stream, const Mlap
         }
         const int njobs = q_prefill_jobs(qp);
         const dim3 g((unsigned)njobs), b(256);
-        switch (q_prefill_token_blocks(p.T)) {
-        case 1: hipLaunchKernelGGL(qproj_prefill_kernel<1>, g, b, 0, stream, qp, njobs); break;
-        case 2: hipLaunchKernelGGL(qproj_prefill_kernel<2>, g, b, 0, stream, qp, njobs); break;
-        default: hipLaunchKernelGGL(qproj_prefill_kernel<4>, g, b, 0, stream, qp, njobs);
+        const int tbk = q_prefill_token_blocks(p.T);
+        if (lip_rider != nullptr) {
+            // the indexer prolog's split projection rides along: one more workgroup per job of a wave pair
+            const LipParams &lp = *lip_rider;
+            const QProj qr = {lp.q_norm, lp.w_qb, lp.qpart, lp.T, lp.q_lora, lp.n_heads, lp.q_norm_scale, lp.w_qb_scale};
+            const int rjobs = lp.n_heads * QPROJ_KSPLIT * ((lp.T + 31) / 32);
+            const dim3 gr((unsigned)(njobs + rjobs));
+            const int steps = lp.q_lora / QPROJ_KSPLIT / 32;
+#define QPF_RIDER(TBV)                                                                                       \
+    switch (steps) {                                                                                         \
+    case 4: hipLaunchKernelGGL((qproj_prefill_kernel<TBV, 2>), gr, b, 0, stream, qp, njobs, qr); break;     \
+    case 8: hipLaunchKernelGGL((qproj_prefill_kernel<TBV, 4>), gr, b, 0, stream, qp, njobs, qr); break;     \
+    case 12: hipLaunchKernelGGL((qproj_prefill_kernel<TBV, 6>), gr, b, 0, stream, qp, njobs, qr); break;    \
+    default: return hipErrorInvalidValue;                                                                    \
+    }
+            if (tbk == 1) { QPF_RIDER(1) } else { QPF_RIDER(2) }
+#undef QPF_RIDER
+            return hipGetLastError();
+        }
+        switch (tbk) {
+        case 1: hipLaunchKernelGGL((qproj_prefill_kernel<1, 0>), g, b, 0, stream, qp, njobs, qp); break;
+        case 2: hipLaunchKernelGGL((qproj_prefill_kernel<2, 0>), g, b, 0, stream, qp, njobs, qp); break;
+        default: hipLaunchKernelGGL((qproj_prefill_kernel<4, 0>), g, b, 0, stream, qp, njobs, qp);
         }
         return hipGetLastError();
     }

@@ -6,8 +6,9 @@
 // workgroups that finish the attention query (absorb product, 70 KB of LDS, four waves) and those that finish the
 // indexer's query rows, key row and weights (54 KB, eight waves) do not depend on each other and fit a compute
 // unit together, so they run side by side instead of one launch after the other.  Where the indexer prolog cannot
-// ride (other than 64 indexer heads) its first launch follows the MLA prolog's third; at prefill sizes every stage
-// has a launch of its own.
+// ride (other than 64 indexer heads) its first launch follows the MLA prolog's third.  Between 9 and 63 tokens the
+// MLA prolog's prefill forms take the jobs of the indexer prolog's first launch along as riders (five launches);
+// from 64 tokens on every stage has a launch of its own.
 #include "prolog_finish.h"
 
 #include "prolog_fused.h"
@@ -55,10 +56,19 @@ hipError_t prolog_fused_launch(const MlapParams &pm, const LipParams &pl, hipStr
                            mla_wgs, q_wgs);
         return hipGetLastError();
     }
-    hipError_t e = mlap_launch_front(pm, stream);
+    // A batch of 9 to 63 tokens: the MLA prolog runs its prefill forms, the indexer prolog its decode forms, and the
+    // jobs of the indexer prolog's first launch (wave jobs with no kind of workgroup of their own) ride in the MLA
+    // prolog's first and third launch, whose workgroups leave half of every compute unit free: five launches, the
+    // last two the finishing stages of the two halves.
+    const bool lip_rides = mlap_takes_lip_rider(pm) && pl.T == pm.T && pl.h == pm.h && pl.q_lora == pm.q_lora && pl.x == pm.x &&
+                           pl.q_norm == pm.q_norm && pl.q_norm_scale == pm.q_norm_scale && !lip_q_on_matrix_cores(pl) &&
+                           !lip_x_on_matrix_cores(pl) && !lip_x_group_rows(pl) && pl.n_heads <= LIP_MAX_HEADS;
+    hipError_t e = mlap_launch_front(pm, stream, nullptr, lip_rides ? &pl : nullptr);
     if (e != hipSuccess) return e;
-    e = lip_launch_linear(pl, stream);
-    if (e != hipSuccess) return e;
+    if (!lip_rides) {
+        e = lip_launch_linear(pl, stream);
+        if (e != hipSuccess) return e;
+    }
     if (mlap_finish_is_prefill(pm) || lip_q_on_matrix_cores(pl)) {
         // prefill sizes: the last stages have forms of their own (the attention query's: one workgroup per compute unit)
         e = mlap_launch_finish(pm, stream);
