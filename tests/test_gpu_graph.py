@@ -116,13 +116,14 @@ def test_prologs_replays_match_eager(b, s1, act, ni):
             assert torch.equal(g_.view(torch.uint8), w_.view(torch.uint8)), f"replay {rep}: output {i} differs from the eager call"
 
 
-def test_fused_prolog_operator_replays_match_the_two_operators_called_eagerly():
+@pytest.mark.parametrize("b,s1,act", [(4, 2, [5000, 300, 129, 64]), (16, 2, [5000, 300, 129, 64] * 4)])
+def test_fused_prolog_operator_replays_match_the_two_operators_called_eagerly(b, s1, act):
     """mla_indexer_prolog_quant_d (one library call, one workspace from torch's pool, the last launches of the two
     halves merged) recorded once and replayed with new hidden states: every replay equals the two separate
-    operators called eagerly on the same inputs, bit for bit."""
+    operators called eagerly on the same inputs, bit for bit.  8 tokens: the decode forms' four launches; 32 tokens:
+    the MLA half's matrix-core forms with the indexer half's first launch riding in them."""
     from pypto_amd.synthetic import gen_indexer_prolog_inputs, gen_mla_prolog_inputs
     dev = torch.device(DEV)
-    b, s1, act = 4, 2, [5000, 300, 129, 64]
     kw = dict(h=512, q_lora_rank=1536)
     mla = gen_mla_prolog_inputs(b, s1, act, seed=31, n_heads=8, **kw).to(dev)
     lip = gen_indexer_prolog_inputs(b, s1, act, seed=32, n_heads=4, **kw).to(dev)
