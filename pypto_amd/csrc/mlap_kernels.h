@@ -101,5 +101,7 @@ int mlap_finish_wgs(const MlapParams &p);
 // launches beside, not inside, its own last launch
 hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream);
 bool mlap_finish_is_prefill(const MlapParams &p);
+// blocks of 32 tokens per workgroup and workgroups of that form's launch
+void mlap_finish_prefill_shape(const MlapParams &p, int &per, int &wgs);
 
 }  // namespace pto

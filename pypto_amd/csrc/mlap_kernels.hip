@@ -393,15 +393,21 @@ __global__ __launch_bounds__(64 * FINP_WAVES) void mlap_finish_prefill_kernel(co
 
 bool mlap_finish_is_prefill(const MlapParams &p) { return mlap_prefill_forms(p); }
 
+void mlap_finish_prefill_shape(const MlapParams &p, int &per, int &wgs)
+{
+    // runs of up to 16 blocks of 32 tokens per workgroup, two runs at least so that 128 heads fill the chip
+    const int nblocks = (p.T + FINP_TOK - 1) / FINP_TOK;
+    per = (nblocks + 1) / 2;
+    per = per > 16 ? 16 : per;
+    wgs = p.n_heads * ((nblocks + per - 1) / per);
+}
+
 hipError_t mlap_launch_finish(const MlapParams &p, hipStream_t stream)
 {
     if (mlap_finish_is_prefill(p)) {
-        // runs of up to 16 blocks of 32 tokens per workgroup, two runs at least so that 128 heads fill the chip
-        const int nblocks = (p.T + FINP_TOK - 1) / FINP_TOK;
-        int per = (nblocks + 1) / 2;
-        per = per > 16 ? 16 : per;
-        const int runs = (nblocks + per - 1) / per;
-        hipLaunchKernelGGL(mlap_finish_prefill_kernel, dim3((unsigned)(p.n_heads * runs)), dim3(64 * FINP_WAVES), 0, stream, p, per);
+        int per, wgs;
+        mlap_finish_prefill_shape(p, per, wgs);
+        hipLaunchKernelGGL(mlap_finish_prefill_kernel, dim3((unsigned)wgs), dim3(64 * FINP_WAVES), 0, stream, p, per);
     } else {
         hipLaunchKernelGGL(mlap_finish_kernel, dim3((unsigned)mlap_finish_wgs(p)), dim3(256), 0, stream, p);
     }

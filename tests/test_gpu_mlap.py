@@ -220,7 +220,8 @@ def run_fused(dm, dl, t, n, n_idx, op=None):
 
 @pytest.mark.parametrize("mode,shape", [("default", "small"), ("exact", "small"), ("matrix_cores", "small"), ("default", "t_512"),
                                         ("default", "t_11_idx_64"), ("exact", "t_11_idx_64"), ("default", "t_3_idx_32"),
-                                        ("default", "t_40_idx_64"), ("exact", "t_40_idx_64"), ("default", "t_7_idx_64")])
+                                        ("default", "t_40_idx_64"), ("exact", "t_40_idx_64"), ("default", "t_7_idx_64"),
+                                        ("default", "t_32_idx_64")])
 def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, shape):
     """150 tokens (ragged last block of the token tiles): the fused operator's prefill-sized launches (unsplit int8
     projections, the attention query's last stage per head and run of token blocks) against the MLA prolog and the
@@ -228,7 +229,8 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, sha
     The two decode-sized shapes: with 64 indexer heads the indexer prolog's first stage rides in the MLA prolog's
     launches (7 tokens by default; 11 in the exact mode: two token groups, the second ragged; 576 hidden channels: a
     second, short group of blocks), with 32 heads it keeps its own launch.  At 40 tokens the MLA half takes its prefill forms by default
-    while the indexer half keeps its decode forms (in the exact mode both keep them, and the rider)."""
+    while the indexer half keeps its decode forms (in the exact mode both keep them, and the rider); at 32 and at 11
+    tokens the two last stages share a launch as well."""
     from pypto_amd import lightning_indexer_prolog_quant_impl as lip_impl
     from pypto_amd import mla_prolog_quant_impl as impl
     from pypto_amd.synthetic import gen_indexer_prolog_inputs
@@ -246,6 +248,9 @@ def test_fused_prolog_at_prefill_size_equals_the_two_operators_chained(mode, sha
     elif shape == "t_40_idx_64":
         kw = dict(h=576, q_lora_rank=512)
         b, s1, act, n_mla, n_idx = 5, 8, [700, 650, 600, 550, 500], 4, 64
+    elif shape == "t_32_idx_64":
+        kw = dict(h=576, q_lora_rank=512)
+        b, s1, act, n_mla, n_idx = 4, 8, [700, 650, 600, 550], 4, 64
     elif shape == "t_3_idx_32":
         kw = dict(h=576, q_lora_rank=512)
         b, s1, act, n_mla, n_idx = 3, 1, [700, 650, 600], 4, 32
