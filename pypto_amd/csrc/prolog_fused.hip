@@ -7,9 +7,8 @@
 // indexer's query rows, key row and weights (54 KB, eight waves) do not depend on each other and fit a compute
 // unit together, so they run side by side instead of one launch after the other.  Where the indexer prolog cannot
 // ride (other than 64 indexer heads) its first launch follows the MLA prolog's third.  Between 9 and 63 tokens the
-// MLA prolog's prefill forms take the jobs of the indexer prolog's first launch along as riders (five launches; four up to 32
-// tokens, where the two last stages share one);
-// from 64 tokens on every stage has a launch of its own.
+// MLA prolog's prefill forms take the jobs of the indexer prolog's first launch along as riders (five launches;
+// four up to 32 tokens, where the two last stages share one); from 64 tokens on every stage has a launch of its own.
 #include "prolog_finish.h"
 
 #include "prolog_fused.h"
