@@ -809,7 +809,7 @@ int pto_mla_indexer_prolog_quant_launch(const PtoMlaIndexerPrologQuantArgs *a, v
     if (rc != PTO_OK) return rc;
     rc = lip_params(&pl.idx, pi);
     if (rc != PTO_OK) return rc;
-    // five launches: the last ones of the two halves do not depend on each other and run as one
+    // four launches up to 32 tokens (the indexer half rides in the MLA half's), five up to 63, six above
     hipError_t e = pto::prolog_fused_launch(pm, pi, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(PTO_E_LAUNCH, "mla_indexer_prolog: launch failed: %s", hipGetErrorString(e));
     return PTO_OK;
